@@ -27,19 +27,28 @@ class KVCacheManager:
         block_size: int = 16,
         device=None,
         dtype=torch.bfloat16,
+        layer_shapes: Optional[List[Optional[tuple]]] = None,
     ):
+        """``layer_shapes`` (optional) gives each layer its own
+        ``(kv_heads, key_dim, value_dim)`` or ``None`` for a layer that keeps no
+        keys (a recurrent layer of a hybrid model); without it every layer gets
+        ``(num_kv_heads, head_dim, head_dim)``."""
         assert block_size & (block_size - 1) == 0, "block_size must be a power of two"
         self.num_layers = num_layers
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.device = device or ("cuda" if torch.cuda.is_available() else "cpu")
+        if layer_shapes is None:
+            layer_shapes = [(num_kv_heads, head_dim, head_dim)] * num_layers
+        assert len(layer_shapes) == num_layers
+        self.layer_shapes = list(layer_shapes)
         self.k_pools = [
-            torch.zeros(num_blocks, block_size, num_kv_heads, head_dim, device=self.device, dtype=dtype)
-            for _ in range(num_layers)
+            None if s is None else torch.zeros(num_blocks, block_size, s[0], s[1], device=self.device, dtype=dtype)
+            for s in layer_shapes
         ]
         self.v_pools = [
-            torch.zeros(num_blocks, block_size, num_kv_heads, head_dim, device=self.device, dtype=dtype)
-            for _ in range(num_layers)
+            None if s is None else torch.zeros(num_blocks, block_size, s[0], s[2], device=self.device, dtype=dtype)
+            for s in layer_shapes
         ]
         self._free: List[int] = list(range(num_blocks - 1, -1, -1))
         self._tables: Dict[int, List[int]] = {}  # seq id -> block ids
@@ -56,6 +65,9 @@ class KVCacheManager:
         return self.blocks_needed(num_tokens) <= self.free_blocks
 
     # ------------------------------------------------------------- allocation
+    def has(self, seq_id) -> bool:
+        return seq_id in self._tables
+
     def allocate(self, seq_id: int, num_tokens: int) -> None:
         need = self.blocks_needed(num_tokens)
         assert need <= self.free_blocks, "KV pool exhausted"

@@ -8,6 +8,13 @@ sequence one token with ``decode_attention_paged`` over the block pools.
 Short requests retire and free their blocks immediately; long prompts
 stream in the moment blocks are available — throughput is bounded by the
 8 TB/s KV stream, not by the longest member of a static batch.
+
+Models that declare ``serves_ragged`` (hybrids of paged attention and
+fixed-size recurrent state) run through one *ragged* step instead:
+``run_ragged`` takes any mix of prompt portions and single decode tokens,
+builds one flat token batch with per-sequence offsets, page tables and state
+slots, and calls the model's ``forward_ragged``. ``step()`` feeds it from the
+chunked-prefill scheduler; a trace replayer can feed it directly.
 """
 
 from typing import Dict, List, Optional, Union
@@ -19,6 +26,8 @@ from .config import GenerationConfig, InferenceConfig
 from .engine import LLMEngine
 from .kv_cache import KVCacheManager
 from .request_manager import Request, RequestManager
+from .state_cache import StateCacheManager
+from ..ops.ragged import RaggedBatch
 
 __all__ = ["ContinuousBatchEngine"]
 
@@ -30,6 +39,7 @@ class ContinuousBatchEngine:
         config: Optional[InferenceConfig] = None,
         num_blocks: Optional[int] = None,
         block_size: int = 16,
+        max_step_tokens: int = 2048,
     ):
         self.config = config or InferenceConfig()
         self.model = model.eval()
@@ -41,6 +51,19 @@ class ContinuousBatchEngine:
             num_blocks = self.config.max_batch_size * (
                 (self.config.max_seq_len + block_size - 1) // block_size
             )
+        self.ragged = bool(getattr(model, "serves_ragged", False))
+        self.max_step_tokens = max_step_tokens
+        self._gen = GenerationConfig()
+        if self.ragged:
+            self.dtype = model.act_dtype
+            shapes = model.kv_layer_shapes()
+            self.kv = KVCacheManager(len(shapes), 0, 0, num_blocks=num_blocks, block_size=block_size,
+                                     device=self.device, dtype=self.dtype, layer_shapes=shapes)
+            self.state = StateCacheManager(model.state_layer_buffers(), self.config.max_batch_size,
+                                           device=self.device)
+            self.rm = RequestManager(self.kv, max_batch_size=self.config.max_batch_size, state=self.state)
+            self._cached: Dict[object, int] = {}  # sequence id -> tokens its caches hold
+            return
         # per-rank layer attributes, not the config: under TP each rank
         # caches only its local KV heads (same rule as LLMEngine)
         attn0 = model.model.layers[0].self_attn
@@ -53,6 +76,76 @@ class ContinuousBatchEngine:
     # -------------------------------------------------------------- requests
     def add_request(self, prompt: List[int], max_new_tokens: Optional[int] = None) -> int:
         return self.rm.add_request(list(prompt), max_new_tokens or self._gen.max_new_tokens)
+
+    # ---------------------------------------------------------- ragged step
+    def open_sequence(self, seq_id) -> None:
+        """Give a sequence a state slot and an (empty) page table."""
+        if not self.kv.has(seq_id):
+            self.kv.allocate(seq_id, 0)
+        self.state.allocate(seq_id)
+        self._cached[seq_id] = 0
+
+    def close_sequence(self, seq_id) -> None:
+        """Return a sequence's pages and state slot."""
+        self.kv.free(seq_id)
+        self.state.free(seq_id)
+        self._cached.pop(seq_id, None)
+
+    @torch.inference_mode()
+    def run_ragged(self, items) -> torch.Tensor:
+        """One ragged engine step. ``items`` is ``[(seq_id, new_tokens, want)]``:
+        the next tokens of open sequences (a prompt portion or one decode
+        token each) and the places among them whose logits are wanted. Returns
+        float32 logits ``[sum(len(want)), vocab]`` in item order; the caches
+        then hold the new tokens."""
+        counts, starts, slots, tables, flat, want = [], [], [], [], [], []
+        at = 0
+        for seq_id, toks, w in items:
+            if seq_id not in self._cached:
+                self.open_sequence(seq_id)
+            s0 = self._cached[seq_id]
+            self.kv.extend(seq_id, s0 + len(toks))
+            counts.append(len(toks))
+            starts.append(s0)
+            slots.append(self.state.slot(seq_id))
+            tables.append(self.kv.table(seq_id))
+            flat += list(toks)
+            want += [at + int(j) for j in w]
+            at += len(toks)
+        assert len(set(slots)) == len(slots), "a sequence appears twice in one step"
+        batch = RaggedBatch.build(counts, starts, slots, self.device, tables, self.kv.block_size)
+        tokens = torch.tensor(flat, dtype=torch.long, device=self.device)
+        widx = torch.tensor(want, dtype=torch.long, device=self.device)
+        logits = self.model.forward_ragged(tokens, batch, self.kv, self.state, widx)
+        for (seq_id, toks, _), s0 in zip(items, starts):
+            self._cached[seq_id] = s0 + len(toks)
+        return logits
+
+    def _step_ragged(self) -> Dict[int, List[int]]:
+        gen, cfg = self._gen, self.config
+        finished: Dict[int, List[int]] = {}
+        plan = self.rm.schedule_chunks(self.max_step_tokens)
+        if not plan:
+            return finished
+        items, samplers = [], []
+        for req, toks in plan:
+            if req.request_id not in self._cached:
+                self._cached[req.request_id] = 0  # the scheduler already took its slot and pages
+            ends = req.num_computed + len(toks) == req.seq_len
+            items.append((req.request_id, toks, [len(toks) - 1] if ends else []))
+            if ends:
+                samplers.append(req)
+        logits = self.run_ragged(items)
+        for req, toks in plan:
+            req.num_computed += len(toks)
+        if samplers:
+            tokens = LLMEngine._sample(logits, gen)
+            for i, req in enumerate(samplers):
+                self.rm.append_token(req, int(tokens[i]), cfg.eos_token_id, cfg.max_seq_len)
+                if req.status.value == "finished":
+                    self._cached.pop(req.request_id, None)
+                    finished[req.request_id] = req.tokens
+        return finished
 
     # --------------------------------------------------------------- forward
     def _forward(self, input_ids, positions, seq_ids, block_tables, seq_lens, prefill):
@@ -91,6 +184,8 @@ class ContinuousBatchEngine:
     def step(self) -> Dict[int, List[int]]:
         """One engine iteration; returns {request_id: full tokens} for
         requests that finished during this step."""
+        if self.ragged:
+            return self._step_ragged()
         gen, cfg = self._gen, self.config
         finished: Dict[int, List[int]] = {}
 

@@ -32,6 +32,7 @@ class Request:
     max_new_tokens: int
     output: List[int] = field(default_factory=list)
     status: RequestStatus = RequestStatus.WAITING
+    num_computed: int = 0  # tokens whose keys / state the caches already hold (chunked prefill)
 
     @property
     def seq_len(self) -> int:
@@ -43,8 +44,9 @@ class Request:
 
 
 class RequestManager:
-    def __init__(self, kv: KVCacheManager, max_batch_size: int = 32):
+    def __init__(self, kv: KVCacheManager, max_batch_size: int = 32, state=None):
         self.kv = kv
+        self.state = state  # optional StateCacheManager: admission then also needs a free state slot
         self.max_batch_size = max_batch_size
         self.waiting: List[Request] = []
         self.running: List[Request] = []
@@ -63,14 +65,36 @@ class RequestManager:
         while self.waiting and len(self.running) < self.max_batch_size:
             req = self.waiting[0]
             worst = len(req.prompt) + req.max_new_tokens
-            if not self.kv.can_allocate(worst):
+            if not self.kv.can_allocate(worst) or (self.state is not None and not self.state.can_allocate()):
                 break
             self.waiting.pop(0)
             self.kv.allocate(req.request_id, len(req.prompt))
+            if self.state is not None:
+                self.state.allocate(req.request_id)
             req.status = RequestStatus.RUNNING
             self.running.append(req)
             admitted.append(req)
         return admitted
+
+    def schedule_chunks(self, max_step_tokens: int):
+        """Chunked-prefill schedule of one ragged step: every running request
+        whose prompt is cached decodes one token; what is left of the token
+        budget goes to prompt portions, oldest request first (newly admitted
+        ones included). Returns ``[(request, tokens_to_run)]``; a request's
+        portion ends at its last known token, whose logits pick the next one."""
+        self.schedule()
+        plan, budget = [], max_step_tokens
+        for req in self.running:
+            if req.seq_len - req.num_computed == 1:
+                plan.append((req, req.tokens[-1:]))
+                budget -= 1
+        for req in self.running:
+            left = req.seq_len - req.num_computed
+            if left > 1 and budget > 0:
+                n = min(left, budget)
+                plan.append((req, req.tokens[req.num_computed : req.num_computed + n]))
+                budget -= n
+        return plan
 
     def append_token(self, req: Request, token: int, eos_token_id: Optional[int], max_seq_len: int) -> None:
         req.output.append(token)
@@ -86,6 +110,8 @@ class RequestManager:
         req.status = RequestStatus.FINISHED
         self.running.remove(req)
         self.kv.free(req.request_id)
+        if self.state is not None:
+            self.state.free(req.request_id)
 
     @property
     def has_work(self) -> bool:

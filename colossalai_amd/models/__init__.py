@@ -3,6 +3,8 @@ from .dit import DIT_CONFIGS, DiT, DiTConfig
 from .deepseek_v3 import DEEPSEEK_V3_CONFIGS, DeepseekV3Config, DeepseekV3ForCausalLM
 from .chatglm2 import CHATGLM_CONFIGS, ChatGLMConfig, ChatGLMForConditionalGeneration
 from .blip2 import Blip2Config, Blip2ForConditionalGeneration
+from .registry import load_pretrained, model_class_for, register_model, registered_models
+from .kipirax import KipiraxConfig, KipiraxForCausalLM
 from .llama import LLAMA_CONFIGS, LlamaConfig, LlamaForCausalLM, llama_flops_per_token
 from .bert import BERT_CONFIGS, BertConfig, BertForMaskedLM, BertForSequenceClassification
 from .opt import OPT_CONFIGS, OPTConfig, OPTForCausalLM
@@ -15,7 +17,9 @@ from .falcon import FALCON_CONFIGS, FalconConfig, FalconForCausalLM
 from .vit import VIT_CONFIGS, ViTConfig, ViTForImageClassification
 from .whisper import WHISPER_CONFIGS, WhisperConfig, WhisperForConditionalGeneration
 
-__all__ = ["LlamaConfig", "LlamaForCausalLM", "LLAMA_CONFIGS", "llama_flops_per_token",
+__all__ = ["load_pretrained", "model_class_for", "register_model", "registered_models",
+           "KipiraxConfig", "KipiraxForCausalLM",
+           "LlamaConfig", "LlamaForCausalLM", "LLAMA_CONFIGS", "llama_flops_per_token",
            "OPTConfig", "OPTForCausalLM", "OPT_CONFIGS",
            "BertConfig", "BertForMaskedLM", "BertForSequenceClassification", "BERT_CONFIGS",
            "T5Config", "T5ForConditionalGeneration", "T5_CONFIGS",

@@ -27,6 +27,8 @@ import torch.nn.functional as F
 
 from ..ops import build_rope_table, fused_add_rms_norm, fused_rope_attention, rms_norm, swiglu
 
+from .registry import register_model
+
 __all__ = ["LlamaConfig", "LlamaForCausalLM", "LLAMA_CONFIGS", "llama_flops_per_token"]
 
 
@@ -487,7 +489,21 @@ class LlamaModel(nn.Module):
         return hidden if is_last else residual
 
 
+@register_model("LlamaForCausalLM", "llama")
 class LlamaForCausalLM(nn.Module):
+    @classmethod
+    def from_checkpoint(cls, config: dict, tensors, dtype=torch.bfloat16, device="cpu"):
+        """Build from an HF-style config.json dict and a name -> tensor mapping
+        (per-projection HF names are packed into the native layout)."""
+        from .hf_compat import load_hf_llama
+
+        keys = ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
+                "num_key_value_heads", "max_position_embeddings", "rms_norm_eps", "rope_theta",
+                "tie_word_embeddings", "attention_bias")
+        model = cls(LlamaConfig(**{k: config[k] for k in keys if k in config})).to(dtype)
+        load_hf_llama(model, dict(tensors), strict=not config.get("tie_word_embeddings", False))
+        return model.to(device).eval()
+
     def __init__(self, cfg: LlamaConfig):
         super().__init__()
         self.config = cfg

@@ -43,3 +43,48 @@ def use_hip(*tensors: torch.Tensor) -> bool:
             f"fall back to eager PyTorch. Build it with `python setup.py build_ext --inplace`. ({_IMPORT_ERROR})"
         )
     return True
+
+
+# ---------------------------------------------------------------------------
+# colossalai_amd._C_serving: the ragged serving kernels (paged attention with
+# window / sinks / distance bias, matrix-state recurrences, short convolution,
+# token shift, grouped norms). It is a separate, small extension so that a
+# fresh checkout that only serves a model compiles these few files and not the
+# training kernels.
+_SERVING = None
+
+
+def build_serving_extension() -> None:
+    """Compile colossalai_amd._C_serving in-tree (gfx950) with the repo's setup.py."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    env = dict(os.environ, PYTORCH_ROCM_ARCH="gfx950", COLOSSALAI_AMD_EXTENSIONS="serving")
+    subprocess.run([sys.executable, "setup.py", "build_ext", "--inplace"], cwd=root, env=env, check=True,
+                   stdout=sys.stderr)
+
+
+def serving_kernels(build_if_missing: bool = True):
+    """Return colossalai_amd._C_serving, compiling it once if it is not built."""
+    global _SERVING
+    if _SERVING is None:
+        import importlib
+
+        try:
+            _SERVING = importlib.import_module("colossalai_amd._C_serving")
+        except ImportError:
+            if not build_if_missing:
+                raise
+            build_serving_extension()
+            importlib.invalidate_caches()
+            _SERVING = importlib.import_module("colossalai_amd._C_serving")
+    return _SERVING
+
+
+def use_serving_hip(*tensors: torch.Tensor) -> bool:
+    """True when the serving ops must take their HIP path (tensors on the GPU);
+    ``serving_kernels()`` then loads, or compiles, the extension — there is no
+    eager fallback on a GPU."""
+    return all(t.is_cuda for t in tensors if isinstance(t, torch.Tensor))

@@ -1,0 +1,71 @@
+"""Grouped RMS normalisation and per-head output normalisation with a gate.
+
+``grouped_rms_norm`` splits the feature axis into ``groups`` equal consecutive
+parts, scales each part by its own ``rsqrt(mean(part^2) + eps)`` and applies an
+element-wise weight; with ``residual`` it adds the result to a float32 residual
+stream in place (norm on the sublayer's *output*). ``groups=1`` is plain RMS
+norm. ``head_rms_norm_gate`` normalises every head vector of a ``[N, H, D]``
+tensor with one shared ``[D]`` weight and optionally multiplies by
+``sigmoid(gate)``. All statistics are float32.
+"""
+
+from typing import Optional
+
+import torch
+
+from ._kernels import serving_kernels, use_serving_hip as use_hip
+
+__all__ = ["grouped_rms_norm", "grouped_rms_norm_ref", "head_rms_norm_gate", "head_rms_norm_gate_ref",
+           "merge_rms_norm", "merge_rms_norm_ref"]
+
+
+def grouped_rms_norm_ref(x, weight, groups: int, eps: float, residual=None, out_dtype=None):
+    shp = x.shape
+    xf = x.float().reshape(*shp[:-1], groups, shp[-1] // groups)
+    y = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).reshape(shp) * weight.float()
+    if residual is not None:
+        residual.add_(y)
+        return residual
+    return y.to(out_dtype or x.dtype)
+
+
+def grouped_rms_norm(x, weight, groups: int, eps: float, residual: Optional[torch.Tensor] = None, out_dtype=None):
+    assert x.shape[-1] % groups == 0, "feature axis must split evenly into the norm groups"
+    if use_hip(x):
+        assert residual is None or residual.dtype == torch.float32
+        return serving_kernels().grouped_rms_norm(x.contiguous(), weight, groups, eps, residual,
+                                                  out_dtype or x.dtype)
+    return grouped_rms_norm_ref(x, weight, groups, eps, residual, out_dtype)
+
+
+def head_rms_norm_gate_ref(x, weight, eps: float, gate=None, out_dtype=None):
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    if gate is not None:
+        y = y * torch.sigmoid(gate.float().reshape(y.shape))
+    return y.to(out_dtype or x.dtype)
+
+
+def head_rms_norm_gate(x, weight, eps: float, gate=None, out_dtype=None):
+    """x [N, H, D] (row-strided allowed), weight [D], gate logits [N, H * D] or None."""
+    if use_hip(x):
+        return serving_kernels().head_rms_norm_gate(x, weight, eps, gate, out_dtype or x.dtype)
+    return head_rms_norm_gate_ref(x, weight, eps, gate, out_dtype)
+
+
+def merge_rms_norm_ref(a, wa, b, wb, eps: float, out_w, groups: int, residual):
+    def unit(t, w):
+        tf = t.float()
+        return tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    m = 0.5 * (unit(a, wa) + unit(b, wb))
+    return grouped_rms_norm_ref(m, out_w, groups, eps, residual)
+
+
+def merge_rms_norm(a, wa, b, wb, eps: float, out_w, groups: int, residual):
+    """Two branch outputs [N, W], each RMS-normed over the full width with its
+    own weight, averaged, then grouped-normed with ``out_w`` and added to the
+    float32 ``residual`` in place — one pass over the row."""
+    if use_hip(a):
+        return serving_kernels().merge_rms_norm(a.contiguous(), wa, b.contiguous(), wb, eps, out_w, groups, residual)
+    return merge_rms_norm_ref(a, wa, b, wb, eps, out_w, groups, residual)

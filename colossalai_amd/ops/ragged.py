@@ -1,0 +1,78 @@
+"""Ragged serving batch descriptor shared by the sequence-state ops.
+
+One engine step runs ``N`` new tokens that belong to ``B`` live sequences:
+a prompt portion of any length next to single decode tokens. Every op that
+carries per-sequence memory (paged keys/values, recurrent matrices, the tail
+of a short convolution, the previous token of a token shift) takes this
+descriptor instead of a dense ``[B, S]`` layout, so that a result never
+depends on how a prompt was cut or on what else shares the step.
+"""
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+
+__all__ = ["RaggedBatch"]
+
+
+@dataclass
+class RaggedBatch:
+    # device tensors (int32)
+    cu: torch.Tensor          # [B + 1] offsets of each sequence's new tokens in the flat token axis
+    start: torch.Tensor       # [B] tokens the sequence already holds (= position of its first new token)
+    slots: torch.Tensor       # [B] state slot of each sequence
+    tok_seq: torch.Tensor     # [N] which sequence (0..B-1) a token belongs to
+    positions: torch.Tensor   # [N] absolute position of a token in its sequence
+    block_tables: Optional[torch.Tensor]  # [B, max_blocks] page ids (None when no layer keeps keys)
+    kv_rows: Optional[torch.Tensor]       # [N] flat pool row (page * page_size + offset) of each token
+    # host mirrors
+    cu_host: List[int]
+    start_host: List[int]
+    slots_host: List[int]
+    page_size: int = 0
+
+    @property
+    def num_seqs(self) -> int:
+        return len(self.start_host)
+
+    @property
+    def num_tokens(self) -> int:
+        return self.cu_host[-1]
+
+    @property
+    def max_new(self) -> int:
+        return max(self.cu_host[i + 1] - self.cu_host[i] for i in range(self.num_seqs))
+
+    @property
+    def max_total(self) -> int:
+        """Longest sequence after this step (cached + new tokens)."""
+        return max(self.start_host[i] + self.cu_host[i + 1] - self.cu_host[i] for i in range(self.num_seqs))
+
+    @classmethod
+    def build(cls, new_counts: Sequence[int], starts: Sequence[int], slots: Sequence[int], device,
+              tables: Optional[Sequence[Sequence[int]]] = None, page_size: int = 0) -> "RaggedBatch":
+        cu = [0]
+        for n in new_counts:
+            assert n > 0, "a sequence in a step brings at least one token"
+            cu.append(cu[-1] + n)
+        tok_seq, pos, rows = [], [], []
+        for i, n in enumerate(new_counts):
+            tok_seq += [i] * n
+            pos += list(range(starts[i], starts[i] + n))
+            if tables is not None:
+                t = tables[i]
+                assert len(t) * page_size >= starts[i] + n, "block table does not cover the new tokens"
+                rows += [t[p // page_size] * page_size + p % page_size for p in range(starts[i], starts[i] + n)]
+        i32 = dict(dtype=torch.int32, device=device)
+        bt = None
+        if tables is not None:
+            width = max(len(t) for t in tables)
+            bt = torch.tensor([list(t) + [0] * (width - len(t)) for t in tables], **i32)
+        return cls(
+            cu=torch.tensor(cu, **i32), start=torch.tensor(list(starts), **i32),
+            slots=torch.tensor(list(slots), **i32), tok_seq=torch.tensor(tok_seq, **i32),
+            positions=torch.tensor(pos, **i32), block_tables=bt,
+            kv_rows=torch.tensor(rows, **i32) if tables is not None else None,
+            cu_host=cu, start_host=list(starts), slots_host=list(slots), page_size=page_size,
+        )

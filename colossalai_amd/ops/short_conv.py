@@ -1,0 +1,38 @@
+"""Short causal depthwise convolution over a ragged serving batch.
+
+``y[t, c] = act(sum_d taps[c, K-1-d] * x[t-d, c])`` for ``d = 0..K-1``, zeros
+ahead of position 0. The last ``K-1`` inputs of a sequence live in ``tail``
+(one ``[K-1, C]`` block per state slot, oldest first) so a portion that starts
+mid-sequence sees the inputs of earlier steps.
+"""
+
+import torch
+import torch.nn.functional as F
+
+from ._kernels import serving_kernels, use_serving_hip as use_hip
+from .ragged import RaggedBatch
+
+__all__ = ["short_conv", "short_conv_ref"]
+
+
+def short_conv_ref(x, taps, tail, batch: RaggedBatch, silu: bool = True):
+    K = taps.shape[1]
+    y = torch.empty_like(x)
+    tf = taps.float()
+    for i in range(batch.num_seqs):
+        lo, hi, slot = batch.cu_host[i], batch.cu_host[i + 1], batch.slots_host[i]
+        hist = tail[slot].float() if batch.start_host[i] > 0 else torch.zeros_like(tail[slot], dtype=torch.float32)
+        full = torch.cat([hist, x[lo:hi].float()], 0)  # [K-1+n, C]
+        acc = torch.zeros(hi - lo, x.shape[1], device=x.device)
+        for j in range(K):
+            acc = acc + full[j : j + hi - lo] * tf[:, j]
+        y[lo:hi] = (F.silu(acc) if silu else acc).to(x.dtype)
+        tail[slot] = full[full.shape[0] - (K - 1):]
+    return y
+
+
+def short_conv(x, taps, tail, batch: RaggedBatch, silu: bool = True):
+    """x [N, C], taps [C, K], tail [slots, K-1, C] float32 (slot-strided allowed)."""
+    if use_hip(x):
+        return serving_kernels().short_conv(x, taps, tail, batch.cu, batch.start, batch.slots, batch.tok_seq, silu)
+    return short_conv_ref(x, taps, tail, batch, silu)
