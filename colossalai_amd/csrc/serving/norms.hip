@@ -1,0 +1,196 @@
+// Normalisation kernels of the serving path (float32 statistics):
+//   grouped_rms_norm   : per-group RMS scaling of a row, optional in-place add
+//                        to the float32 residual stream;
+//   head_rms_norm_gate : per-head RMS norm of [N, H, D] with a shared [D]
+//                        weight and an optional sigmoid gate;
+//   merge_rms_norm     : two branch rows, each full-width RMS-normed with its
+//                        own weight, averaged, group-normed and added to the
+//                        residual — one pass, the merged row staged in LDS.
+#include "serving_common.h"
+
+namespace cai {
+namespace serving {
+
+// One wave per (row, group).
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void grouped_rms_norm_kernel(
+    TO* __restrict__ out, float* __restrict__ residual, const TI* __restrict__ x, const float* __restrict__ w,
+    long units, int groups, int gs, float eps) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= units) return;
+  const long row = unit / groups;
+  const int g = (int)(unit % groups);
+  const long base = (row * groups + g) * (long)gs;
+  float ssq = 0.0f;
+  for (int i = lane; i < gs; i += 64) {
+    const float v = ldf(x + base + i);
+    ssq += v * v;
+  }
+  ssq = wave_reduce_sum(ssq);
+  const float inv = 1.0f / sqrtf(ssq / (float)gs + eps);
+  for (int i = lane; i < gs; i += 64) {
+    const float y = ldf(x + base + i) * inv * w[g * gs + i];
+    if (residual != nullptr) residual[base + i] += y;
+    else stf(out + base + i, y);
+  }
+}
+
+at::Tensor grouped_rms_norm(at::Tensor x, at::Tensor weight, int64_t groups, double eps,
+                            c10::optional<at::Tensor> residual, at::ScalarType out_dtype) {
+  check_act(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x must be contiguous [N, W]");
+  const long N = x.size(0);
+  const int W = (int)x.size(1);
+  TORCH_CHECK(groups > 0 && W % groups == 0);
+  at::Tensor w = f32c(weight);
+  TORCH_CHECK(w.numel() == W);
+  float* res = nullptr;
+  at::Tensor out;
+  if (residual.has_value()) {
+    TORCH_CHECK(is_f32(*residual) && residual->is_contiguous() && residual->sizes() == x.sizes(),
+                "residual must be contiguous float32 of x's shape");
+    res = residual->data_ptr<float>();
+    out = *residual;
+  } else {
+    out = at::empty({N, W}, x.options().dtype(out_dtype));
+  }
+  if (N == 0) return out;
+  const long units = N * groups;
+  const unsigned grid = (unsigned)((units + 3) / 4);
+  SERVING_DISPATCH_ACT(x, TI, {
+    if (res != nullptr) {
+      hipLaunchKernelGGL((grouped_rms_norm_kernel<TI, float>), dim3(grid), dim3(256), 0, stream(), (float*)nullptr, res,
+                         ptr<TI>(x), w.data_ptr<float>(), units, (int)groups, W / (int)groups, (float)eps);
+    } else {
+      SERVING_DISPATCH_ACT(out, TO, {
+        hipLaunchKernelGGL((grouped_rms_norm_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream(), ptr<TO>(out),
+                           (float*)nullptr, ptr<TI>(x), w.data_ptr<float>(), units, (int)groups, W / (int)groups,
+                           (float)eps);
+      });
+    }
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
+// One wave per (n, h). x row-strided: element (n, h, d) at n*xs + h*D + d.
+template <typename TI, typename TG, typename TO>
+__global__ __launch_bounds__(256) void head_rms_norm_gate_kernel(
+    TO* __restrict__ out, const TI* __restrict__ x, long xs, const float* __restrict__ w, const TG* __restrict__ gate,
+    long gs, long units, int H, int D, float eps) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= units) return;
+  const long n = unit / H;
+  const int h = (int)(unit % H);
+  const TI* xr = x + n * xs + (long)h * D;
+  float ssq = 0.0f;
+  for (int i = lane; i < D; i += 64) {
+    const float v = ldf(xr + i);
+    ssq += v * v;
+  }
+  ssq = wave_reduce_sum(ssq);
+  const float inv = 1.0f / sqrtf(ssq / (float)D + eps);
+  for (int i = lane; i < D; i += 64) {
+    float y = ldf(xr + i) * inv * w[i];
+    if (gate != nullptr) y *= sigmoidf_(ldf(gate + n * gs + (long)h * D + i));
+    stf(out + (n * H + h) * (long)D + i, y);
+  }
+}
+
+at::Tensor head_rms_norm_gate(at::Tensor x, at::Tensor weight, double eps, c10::optional<at::Tensor> gate,
+                              at::ScalarType out_dtype) {
+  check_act(x, "x");
+  TORCH_CHECK(x.dim() == 3 && x.stride(2) == 1 && x.stride(1) == x.size(2), "x must be [N, H, D] with dense rows");
+  const long N = x.size(0);
+  const int H = (int)x.size(1), D = (int)x.size(2);
+  at::Tensor w = f32c(weight);
+  TORCH_CHECK(w.numel() == D);
+  at::Tensor out = at::empty({N, H, D}, x.options().dtype(out_dtype));
+  if (N == 0) return out;
+  long gs = 0;
+  if (gate.has_value()) {
+    check_act(*gate, "gate");
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == N && gate->size(1) == (long)H * D && gate->stride(1) == 1);
+    gs = gate->stride(0);
+  }
+  const long units = N * H;
+  const unsigned grid = (unsigned)((units + 3) / 4);
+  SERVING_DISPATCH_ACT(x, TI, {
+    SERVING_DISPATCH_ACT(out, TO, {
+      if (gate.has_value()) {
+        SERVING_DISPATCH_ACT(*gate, TG, {
+          hipLaunchKernelGGL((head_rms_norm_gate_kernel<TI, TG, TO>), dim3(grid), dim3(256), 0, stream(), ptr<TO>(out),
+                             ptr<TI>(x), (long)x.stride(0), w.data_ptr<float>(), ptr<TG>(*gate), gs, units, H, D,
+                             (float)eps);
+        });
+      } else {
+        hipLaunchKernelGGL((head_rms_norm_gate_kernel<TI, float, TO>), dim3(grid), dim3(256), 0, stream(),
+                           ptr<TO>(out), ptr<TI>(x), (long)x.stride(0), w.data_ptr<float>(), (const float*)nullptr,
+                           0L, units, H, D, (float)eps);
+      }
+    });
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
+// One block per row; the merged row lives in LDS (W floats).
+template <typename T>
+__global__ __launch_bounds__(256) void merge_rms_norm_kernel(
+    float* __restrict__ residual, const T* __restrict__ a, const float* __restrict__ wa, const T* __restrict__ b,
+    const float* __restrict__ wb, const float* __restrict__ wo, int W, int groups, float eps) {
+  extern __shared__ float merged[];
+  __shared__ float red[8];
+  const long row = blockIdx.x;
+  const T* ar = a + row * W;
+  const T* br = b + row * W;
+  float sa = 0.0f, sb = 0.0f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float va = ldf(ar + i), vb = ldf(br + i);
+    sa += va * va;
+    sb += vb * vb;
+  }
+  sa = block_reduce_sum(sa, red);
+  sb = block_reduce_sum(sb, red);
+  const float ia = 1.0f / sqrtf(sa / (float)W + eps), ib = 1.0f / sqrtf(sb / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    merged[i] = 0.5f * (ldf(ar + i) * ia * wa[i] + ldf(br + i) * ib * wb[i]);
+  __syncthreads();
+  const int gs = W / groups, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  for (int g = threadIdx.x >> 6; g < groups; g += nw) {
+    float s = 0.0f;
+    for (int i = lane; i < gs; i += 64) {
+      const float v = merged[g * gs + i];
+      s += v * v;
+    }
+    s = wave_reduce_sum(s);
+    const float inv = 1.0f / sqrtf(s / (float)gs + eps);
+    for (int i = lane; i < gs; i += 64) residual[row * W + g * gs + i] += merged[g * gs + i] * inv * wo[g * gs + i];
+  }
+}
+
+at::Tensor merge_rms_norm(at::Tensor a, at::Tensor wa, at::Tensor b, at::Tensor wb, double eps, at::Tensor out_w,
+                          int64_t groups, at::Tensor residual) {
+  check_act(a, "a");
+  TORCH_CHECK(a.dim() == 2 && a.is_contiguous() && b.is_contiguous() && a.sizes() == b.sizes() &&
+              a.scalar_type() == b.scalar_type());
+  TORCH_CHECK(is_f32(residual) && residual.is_contiguous() && residual.sizes() == a.sizes());
+  const long N = a.size(0);
+  const int W = (int)a.size(1);
+  TORCH_CHECK(groups > 0 && W % groups == 0 && W * 4 <= 64 * 1024, "row too wide for the LDS-staged merge");
+  at::Tensor fa = f32c(wa), fb = f32c(wb), fo = f32c(out_w);
+  TORCH_CHECK(fa.numel() == W && fb.numel() == W && fo.numel() == W);
+  if (N == 0) return residual;
+  SERVING_DISPATCH_ACT(a, T, {
+    hipLaunchKernelGGL(merge_rms_norm_kernel<T>, dim3((unsigned)N), dim3(256), (size_t)W * 4, stream(),
+                       residual.data_ptr<float>(), ptr<T>(a), fa.data_ptr<float>(), ptr<T>(b), fb.data_ptr<float>(),
+                       fo.data_ptr<float>(), W, (int)groups, (float)eps);
+  });
+  HIP_CHECK_LAST();
+  return residual;
+}
+
+}  // namespace serving
+}  // namespace cai

@@ -1,0 +1,266 @@
+// Matrix-state linear recurrences over a ragged batch (float32 state).
+//
+// Each head keeps S [D, Dv] per state slot. Columns of S (value channels) are
+// independent in both update rules, so a value channel is owned by P adjacent
+// lanes that split the D rows between them (16 rows per lane, in registers);
+// the two dot products per token are reduced across those P lanes. A wave
+// walks its sequence's new tokens in order, so prompt portions and single
+// decode tokens are the same code, and the state only touches memory at the
+// start and the end of a portion: cutting a prompt differently cannot change
+// a result.
+//
+//   delta: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
+//   tied : S <- diag(f) S + (1 - f) v^T;                          o = S^T q
+//
+// A prologue kernel turns the raw projections into float32 operands once per
+// token (unit-length q/k, decay from its logits, gates), so the sequential
+// loop holds no transcendental.
+#include "serving_common.h"
+
+namespace cai {
+namespace serving {
+
+constexpr int DPL = 16;  // rows of S per lane
+
+// ------------------------------------------------------------------ prologue
+// One block per token. q/k [N, G, D] row-strided; dt [N, H*D] row-strided.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(
+    float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ dec, float* __restrict__ beta,
+    const T* __restrict__ q, long qs, const T* __restrict__ k, long ks, const T* __restrict__ bl, long bs,
+    const T* __restrict__ dt, long ds, const float* __restrict__ A_log, const float* __restrict__ dt_bias, int G, int H,
+    int D, float unit_eps, float q_scale) {
+  const long n = blockIdx.x;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int u = wid; u < 2 * G; u += nw) {
+    const bool isq = u < G;
+    const int g = isq ? u : u - G;
+    const T* src = (isq ? q + n * qs : k + n * ks) + (long)g * D;
+    float ssq = 0.0f;
+    for (int i = lane; i < D; i += 64) {
+      const float v = ldf(src + i);
+      ssq += v * v;
+    }
+    ssq = wave_reduce_sum(ssq);
+    const float inv = (1.0f / sqrtf(ssq + unit_eps)) * (isq ? q_scale : 1.0f);
+    float* dst = (isq ? qn : kn) + (n * G + g) * (long)D;
+    for (int i = lane; i < D; i += 64) dst[i] = ldf(src + i) * inv;
+  }
+  const int HD = H * D;
+  for (int i = threadIdx.x; i < HD; i += blockDim.x) {
+    const float a = expf(A_log[i / D]);
+    dec[n * HD + i] = expf(-a * softplusf_(ldf(dt + n * ds + i) + dt_bias[i]));
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) beta[n * H + h] = sigmoidf_(ldf(bl + n * bs + h));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tied_prepare_kernel(
+    float* __restrict__ qa, float* __restrict__ f, const T* __restrict__ q, long qs, const T* __restrict__ fl, long fs,
+    const float* __restrict__ f_bias, const float* __restrict__ lower, int HD) {
+  const long n = blockIdx.x;
+  for (int i = threadIdx.x; i < HD; i += blockDim.x) {
+    const float qv = ldf(q + n * qs + i);
+    qa[n * HD + i] = qv * sigmoidf_(qv);
+    const float lo = lower[i];
+    f[n * HD + i] = lo + (1.0f - lo) * sigmoidf_(ldf(fl + n * fs + i) + f_bias[i]);
+  }
+}
+
+// ---------------------------------------------------------------------- scan
+DEV_INLINE void load_rows(float* dst, const float* base, int d0, int D, bool vec, float fill) {
+  if (vec && d0 + DPL <= D) {
+#pragma unroll
+    for (int j = 0; j < DPL; j += 4) {
+      const float4v t = *reinterpret_cast<const float4v*>(base + d0 + j);
+      dst[j] = t[0]; dst[j + 1] = t[1]; dst[j + 2] = t[2]; dst[j + 3] = t[3];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) dst[j] = (d0 + j < D) ? base[d0 + j] : fill;
+  }
+}
+
+template <int P>
+DEV_INLINE float reduce_p(float v) {
+#pragma unroll
+  for (int off = 1; off < P; off <<= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+// grid (ceil(Dv / (64 / P)), H, B), one wave per block.
+// q, k: [N, Hq, D] float (Hq = H / rep); gate: [N, H, D] float (decay g or forget f).
+template <int P, bool DELTA, typename TV>
+__global__ __launch_bounds__(64) void matrix_state_scan_kernel(
+    float* __restrict__ out, const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ gate,
+    const float* __restrict__ beta, const TV* __restrict__ v, long vs, float* __restrict__ state, long ss,
+    const int* __restrict__ cu, const int* __restrict__ start, const int* __restrict__ slots, int H, int rep, int D,
+    int Dv) {
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int p = lane % P;
+  const int c = blockIdx.x * (64 / P) + lane / P;
+  const bool live = c < Dv;
+  const int cc = live ? c : Dv - 1;
+  const int d0 = p * DPL;
+  const int Hq = H / rep, hq = h / rep;
+  const bool vec = (D % 4) == 0;
+  const int t0 = cu[b], t1 = cu[b + 1];
+  float* Sg = state + (long)slots[b] * ss + (long)h * D * Dv;
+
+  float S[DPL];
+  const bool fresh = start[b] == 0;
+#pragma unroll
+  for (int j = 0; j < DPL; ++j) S[j] = (!fresh && d0 + j < D) ? Sg[(long)(d0 + j) * Dv + cc] : 0.0f;
+
+  float qn[DPL], kn[DPL], gn[DPL], vn, bn = 0.0f;
+  // operands of the first token
+  load_rows(qn, q + ((long)t0 * Hq + hq) * D, d0, D, vec, 0.0f);
+  if (DELTA) load_rows(kn, k + ((long)t0 * Hq + hq) * D, d0, D, vec, 0.0f);
+  load_rows(gn, gate + ((long)t0 * H + h) * D, d0, D, vec, 1.0f);
+  vn = ldf(v + (long)t0 * vs + (long)h * Dv + cc);
+  if (DELTA) bn = beta[(long)t0 * H + h];
+
+  for (int t = t0; t < t1; ++t) {
+    float qc[DPL], kc[DPL], gc[DPL];
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) { qc[j] = qn[j]; gc[j] = gn[j]; if (DELTA) kc[j] = kn[j]; }
+    const float vc = vn, bc = bn;
+    if (t + 1 < t1) {  // fetch the next token's operands while this one computes
+      load_rows(qn, q + ((long)(t + 1) * Hq + hq) * D, d0, D, vec, 0.0f);
+      if (DELTA) load_rows(kn, k + ((long)(t + 1) * Hq + hq) * D, d0, D, vec, 0.0f);
+      load_rows(gn, gate + ((long)(t + 1) * H + h) * D, d0, D, vec, 1.0f);
+      vn = ldf(v + (long)(t + 1) * vs + (long)h * Dv + cc);
+      if (DELTA) bn = beta[(long)(t + 1) * H + h];
+    }
+    float o = 0.0f;
+    if (DELTA) {
+      float dot = 0.0f;
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) {
+        S[j] *= gc[j];
+        dot += S[j] * kc[j];
+      }
+      dot = reduce_p<P>(dot);
+      const float u = bc * (vc - dot);
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) {
+        S[j] += kc[j] * u;
+        o += S[j] * qc[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < DPL; ++j) {
+        S[j] = gc[j] * S[j] + (1.0f - gc[j]) * vc;
+        o += S[j] * qc[j];
+      }
+    }
+    o = reduce_p<P>(o);
+    if (p == 0 && live) out[((long)t * H + h) * Dv + c] = o;
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < DPL; ++j)
+      if (d0 + j < D) Sg[(long)(d0 + j) * Dv + c] = S[j];
+  }
+}
+
+template <bool DELTA, typename TV>
+static void launch_scan(float* out, const float* q, const float* k, const float* gate, const float* beta, const TV* v,
+                        long vs, float* state, long ss, const int* cu, const int* start, const int* slots, int B,
+                        int H, int rep, int D, int Dv) {
+  int P = 1;
+  while (P * DPL < D) P <<= 1;
+  TORCH_CHECK(P <= 16, "key size above 256 is not supported by the recurrence kernel");
+  const dim3 grid((unsigned)((Dv + 64 / P - 1) / (64 / P)), (unsigned)H, (unsigned)B);
+#define SCAN_CASE(PP)                                                                                              \
+  case PP:                                                                                                         \
+    hipLaunchKernelGGL((matrix_state_scan_kernel<PP, DELTA, TV>), grid, dim3(64), 0, stream(), out, q, k, gate,    \
+                       beta, v, vs, state, ss, cu, start, slots, H, rep, D, Dv);                                   \
+    break;
+  switch (P) {
+    SCAN_CASE(1) SCAN_CASE(2) SCAN_CASE(4) SCAN_CASE(8) SCAN_CASE(16)
+  }
+#undef SCAN_CASE
+  HIP_CHECK_LAST();
+}
+
+static void check_state(const at::Tensor& state, int H, int D, int Dv) {
+  TORCH_CHECK(state.is_cuda() && is_f32(state) && state.dim() == 4 && state.size(1) == H && state.size(2) == D &&
+              state.size(3) == Dv && state.stride(3) == 1 && state.stride(2) == Dv && state.stride(1) == (long)D * Dv,
+              "state must be float32 [slots, H, D, Dv], dense inside a slot");
+}
+
+static void check_rows3(const at::Tensor& t, const char* name) {
+  check_act(t, name);
+  TORCH_CHECK(t.dim() == 3 && t.stride(2) == 1 && t.stride(1) == t.size(2), name, " must be [N, heads, dim] with dense rows");
+}
+
+at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta_logit, at::Tensor dt,
+                            at::Tensor A_log, at::Tensor dt_bias, at::Tensor state, at::Tensor cu, at::Tensor start,
+                            at::Tensor slots, double unit_eps, double q_scale) {
+  check_rows3(q, "q"); check_rows3(k, "k"); check_rows3(v, "v");
+  check_act(beta_logit, "beta_logit"); check_act(dt, "dt");
+  const long N = q.size(0);
+  const int G = (int)q.size(1), D = (int)q.size(2), H = (int)v.size(1), Dv = (int)v.size(2);
+  TORCH_CHECK(k.size(0) == N && v.size(0) == N && k.size(1) == G && k.size(2) == D && H % G == 0);
+  TORCH_CHECK(beta_logit.dim() == 2 && beta_logit.size(0) == N && beta_logit.size(1) == H && beta_logit.stride(1) == 1);
+  TORCH_CHECK(dt.dim() == 2 && dt.size(0) == N && dt.size(1) == (long)H * D && dt.stride(1) == 1);
+  TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type() &&
+              q.scalar_type() == beta_logit.scalar_type() && q.scalar_type() == dt.scalar_type());
+  check_state(state, H, D, Dv);
+  check_i32(cu, "cu"); check_i32(start, "start"); check_i32(slots, "slots");
+  const int B = (int)start.numel();
+  at::Tensor Af = f32c(A_log), bf = f32c(dt_bias);
+  TORCH_CHECK(Af.numel() == H && bf.numel() == (long)H * D);
+  auto fo = q.options().dtype(at::kFloat);
+  at::Tensor out = at::empty({N, H, Dv}, fo);
+  if (N == 0) return out;
+  at::Tensor qn = at::empty({N, G, D}, fo), kn = at::empty({N, G, D}, fo), dec = at::empty({N, H, D}, fo),
+             beta = at::empty({N, H}, fo);
+  SERVING_DISPATCH_ACT(q, T, {
+    hipLaunchKernelGGL(delta_prepare_kernel<T>, dim3((unsigned)N), dim3(256), 0, stream(), qn.data_ptr<float>(),
+                       kn.data_ptr<float>(), dec.data_ptr<float>(), beta.data_ptr<float>(), ptr<T>(q),
+                       (long)q.stride(0), ptr<T>(k), (long)k.stride(0), ptr<T>(beta_logit), (long)beta_logit.stride(0),
+                       ptr<T>(dt), (long)dt.stride(0), Af.data_ptr<float>(), bf.data_ptr<float>(), G, H, D,
+                       (float)unit_eps, (float)q_scale);
+    HIP_CHECK_LAST();
+    launch_scan<true, T>(out.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(), dec.data_ptr<float>(),
+                         beta.data_ptr<float>(), ptr<T>(v), (long)v.stride(0), state.data_ptr<float>(),
+                         (long)state.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(), B, H,
+                         H / G, D, Dv);
+  });
+  return out;
+}
+
+at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, at::Tensor f_bias, at::Tensor lower,
+                                at::Tensor state, at::Tensor cu, at::Tensor start, at::Tensor slots) {
+  check_rows3(q, "q"); check_rows3(f_logit, "f_logit"); check_rows3(v, "v");
+  const long N = q.size(0);
+  const int H = (int)q.size(1), D = (int)q.size(2), Dv = (int)v.size(2);
+  TORCH_CHECK(f_logit.sizes() == q.sizes() && v.size(0) == N && v.size(1) == H);
+  TORCH_CHECK(q.scalar_type() == f_logit.scalar_type() && q.scalar_type() == v.scalar_type());
+  check_state(state, H, D, Dv);
+  check_i32(cu, "cu"); check_i32(start, "start"); check_i32(slots, "slots");
+  const int B = (int)start.numel();
+  at::Tensor fb = f32c(f_bias), lo = f32c(lower);
+  TORCH_CHECK(fb.numel() == (long)H * D && lo.numel() == (long)H * D);
+  auto fo = q.options().dtype(at::kFloat);
+  at::Tensor out = at::empty({N, H, Dv}, fo);
+  if (N == 0) return out;
+  at::Tensor qa = at::empty({N, H, D}, fo), f = at::empty({N, H, D}, fo);
+  SERVING_DISPATCH_ACT(q, T, {
+    hipLaunchKernelGGL(tied_prepare_kernel<T>, dim3((unsigned)N), dim3(256), 0, stream(), qa.data_ptr<float>(),
+                       f.data_ptr<float>(), ptr<T>(q), (long)q.stride(0), ptr<T>(f_logit), (long)f_logit.stride(0),
+                       fb.data_ptr<float>(), lo.data_ptr<float>(), H * D);
+    HIP_CHECK_LAST();
+    launch_scan<false, T>(out.data_ptr<float>(), qa.data_ptr<float>(), (const float*)nullptr, f.data_ptr<float>(),
+                          (const float*)nullptr, ptr<T>(v), (long)v.stride(0), state.data_ptr<float>(),
+                          (long)state.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(), B, H,
+                          1, D, Dv);
+  });
+  return out;
+}
+
+}  // namespace serving
+}  // namespace cai

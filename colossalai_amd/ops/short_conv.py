@@ -21,13 +21,19 @@ def short_conv_ref(x, taps, tail, batch: RaggedBatch, silu: bool = True):
     tf = taps.float()
     for i in range(batch.num_seqs):
         lo, hi, slot = batch.cu_host[i], batch.cu_host[i + 1], batch.slots_host[i]
-        hist = tail[slot].float() if batch.start_host[i] > 0 else torch.zeros_like(tail[slot], dtype=torch.float32)
+        if K == 1:
+            hist = x.new_zeros(0, x.shape[1], dtype=torch.float32)
+        elif batch.start_host[i] > 0:
+            hist = tail[slot].float()
+        else:
+            hist = torch.zeros_like(tail[slot], dtype=torch.float32)
         full = torch.cat([hist, x[lo:hi].float()], 0)  # [K-1+n, C]
         acc = torch.zeros(hi - lo, x.shape[1], device=x.device)
         for j in range(K):
             acc = acc + full[j : j + hi - lo] * tf[:, j]
         y[lo:hi] = (F.silu(acc) if silu else acc).to(x.dtype)
-        tail[slot] = full[full.shape[0] - (K - 1):]
+        if K > 1:
+            tail[slot] = full[full.shape[0] - (K - 1):]
     return y
 
 

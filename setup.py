@@ -20,6 +20,12 @@ CSRC_CPU = os.path.join(THIS_DIR, "colossalai_amd", "csrc_cpu")
 sources = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".cpp")) and not f.endswith("_hip.hip")]
 cpu_sources = [os.path.join(CSRC_CPU, f) for f in sorted(os.listdir(CSRC_CPU)) if f.endswith(".cpp")]
 
+SERVING = os.path.join(CSRC, "serving")
+serving_sources = [os.path.join(SERVING, f) for f in sorted(os.listdir(SERVING))
+                   if f.endswith((".hip", ".cpp")) and not f.endswith("_hip.hip")]
+# -packed-fp32-ops off: the compiler then emits no packed float32 arithmetic
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
 ext = CUDAExtension(
     name="colossalai_amd._C",
     sources=sources,
@@ -30,7 +36,18 @@ ext = CUDAExtension(
             "-std=c++17",
             "--offload-arch=gfx950",
             "-fgpu-flush-denormals-to-zero",
-        ],
+        ] + NO_PACKED_FP32,
+    },
+)
+
+# the ragged serving kernels: a small extension of their own, so that serving a
+# model from a fresh checkout compiles these files only
+serving_ext = CUDAExtension(
+    name="colossalai_amd._C_serving",
+    sources=serving_sources,
+    extra_compile_args={
+        "cxx": ["-O3", "-std=c++17"],
+        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"] + NO_PACKED_FP32,
     },
 )
 
@@ -45,6 +62,8 @@ setup(
     name="colossalai_amd",
     version="0.1.0",
     packages=find_packages(include=["colossalai_amd", "colossalai_amd.*"]),
-    ext_modules=[ext, cpu_ext],
+    # COLOSSALAI_AMD_EXTENSIONS=serving builds just the serving kernels
+    ext_modules=[serving_ext] if os.environ.get("COLOSSALAI_AMD_EXTENSIONS") == "serving"
+    else [ext, cpu_ext, serving_ext],
     cmdclass={"build_ext": BuildExtension.with_options(use_ninja=True)},
 )

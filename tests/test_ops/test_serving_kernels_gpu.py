@@ -1,0 +1,170 @@
+"""HIP serving kernels against their float32 PyTorch references (same op,
+run on CPU copies of the inputs): ragged batches that mix fresh sequences,
+continued sequences and single decode tokens, in bfloat16 and float32."""
+
+import pytest
+import torch
+
+from colossalai_amd.ops import group_norm, linear_recurrence, paged_attention, short_conv, token_shift
+from colossalai_amd.ops.activation import relu_squared, softcap
+from colossalai_amd.ops.ragged import RaggedBatch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def make_batch(device, page=16):
+    # a fresh prompt, a continued portion, two decode tokens (one at a page border), a fresh single token
+    counts = [37, 5, 1, 1, 1]
+    starts = [0, 21, 63, 64, 0]
+    slots = [3, 0, 5, 1, 4]
+    tables, nxt = [], 0
+    for c, s in zip(counts, starts):
+        need = (c + s + page - 1) // page
+        tables.append(list(range(nxt + need - 1, nxt - 1, -1)))  # pages in descending order: not contiguous
+        nxt += need
+    return (RaggedBatch.build(counts, starts, slots, device, tables, page),
+            RaggedBatch.build(counts, starts, slots, "cpu", tables, page), nxt)
+
+
+def both(t):
+    return t.cuda(), t.clone()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_token_shift(dtype):
+    torch.manual_seed(0)
+    gb, cb, _ = make_batch("cuda")
+    W = 200
+    x = torch.randn(gb.num_tokens, W)
+    mu = torch.rand(W)
+    arena = torch.randn(6, W + 8)
+    pg, pc = arena.cuda()[:, 4 : 4 + W], arena.clone()[:, 4 : 4 + W]
+    out = token_shift.token_shift(x.cuda(), mu.cuda(), pg, gb, dtype)
+    ref = token_shift.token_shift_ref(x, mu, pc, cb, dtype)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **tol(dtype))
+    torch.testing.assert_close(pg.cpu(), pc)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("groups,W", [(1, 96), (4, 320), (3, 600)])
+def test_grouped_rms_norm(dtype, groups, W):
+    torch.manual_seed(1)
+    x = torch.randn(19, W).to(dtype)
+    w = torch.randn(W)
+    out = group_norm.grouped_rms_norm(x.cuda(), w.cuda(), groups, 1e-5)
+    torch.testing.assert_close(out.cpu().float(), group_norm.grouped_rms_norm_ref(x, w, groups, 1e-5).float(), **tol(dtype))
+    res = torch.randn(19, W)
+    rg = res.cuda()
+    group_norm.grouped_rms_norm(x.cuda(), w.cuda(), groups, 1e-5, rg)
+    group_norm.grouped_rms_norm_ref(x, w, groups, 1e-5, res)
+    torch.testing.assert_close(rg.cpu(), res, rtol=2e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_head_norm_gate_and_merge(dtype):
+    torch.manual_seed(2)
+    N, H, D, pad = 11, 3, 40, 8
+    wide = torch.randn(N, H * D + pad).to(dtype)
+    gate = torch.randn(N, H * D + pad).to(dtype)
+    w = torch.randn(D)
+    out = group_norm.head_rms_norm_gate(wide.cuda()[:, : H * D].view(N, H, D), w.cuda(), 1e-6,
+                                        gate.cuda()[:, pad:], torch.float32)
+    ref = group_norm.head_rms_norm_gate_ref(wide[:, : H * D].view(N, H, D), w, 1e-6, gate[:, pad:], torch.float32)
+    torch.testing.assert_close(out.cpu(), ref, **tol(dtype))
+    W = 120
+    a, b = torch.randn(N, W).to(dtype), (torch.randn(N, W) * 3).to(dtype)
+    wa, wb, wo = torch.randn(W), torch.randn(W), torch.randn(W)
+    res = torch.randn(N, W)
+    rg = res.cuda()
+    group_norm.merge_rms_norm(a.cuda(), wa.cuda(), b.cuda(), wb.cuda(), 1e-6, wo.cuda(), 3, rg)
+    group_norm.merge_rms_norm_ref(a, wa, b, wb, 1e-6, wo, 3, res)
+    torch.testing.assert_close(rg.cpu(), res, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("K", [1, 2, 4, 7])
+def test_short_conv(dtype, K):
+    torch.manual_seed(3)
+    gb, cb, _ = make_batch("cuda")
+    C, pad = 72, 5
+    wide = torch.randn(gb.num_tokens, C + pad).to(dtype)
+    taps = torch.randn(C, K)
+    arena = torch.randn(6, max(K - 1, 1) * C + 4)
+    tg = arena.cuda()[:, : (K - 1) * C].view(6, K - 1, C) if K > 1 else None
+    tc = arena.clone()[:, : (K - 1) * C].view(6, K - 1, C) if K > 1 else None
+    out = short_conv.short_conv(wide.cuda()[:, :C], taps.cuda(), tg, gb, True)
+    ref = short_conv.short_conv_ref(wide[:, :C], taps, tc, cb, True)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **tol(dtype))
+    if K > 1:
+        torch.testing.assert_close(tg.cpu(), tc, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 24), (3, 3, 20, 64), (2, 1, 128, 70), (2, 2, 8, 8)])
+def test_gated_delta_rule(dtype, H, G, D, Dv):
+    torch.manual_seed(4)
+    gb, cb, _ = make_batch("cuda")
+    N = gb.num_tokens
+    q, k, v = (torch.randn(N, G, D).to(dtype), torch.randn(N, G, D).to(dtype), torch.randn(N, H, Dv).to(dtype))
+    bl, dt = torch.randn(N, H).to(dtype), torch.randn(N, H * D).to(dtype)
+    A, bias = torch.randn(H) - 1, torch.randn(H * D)
+    state = torch.randn(6, H, D, Dv)
+    sg = state.cuda()
+    out = linear_recurrence.gated_delta_rule(q.cuda(), k.cuda(), v.cuda(), bl.cuda(), dt.cuda(), A.cuda(), bias.cuda(),
+                                             sg, gb, 1e-6, D ** -0.5)
+    ref = linear_recurrence.gated_delta_rule_ref(q, k, v, bl, dt, A, bias, state, cb, 1e-6, D ** -0.5)
+    torch.testing.assert_close(out.cpu(), ref, rtol=2e-4, atol=2e-4)
+    live = sorted(gb.slots_host)
+    torch.testing.assert_close(sg.cpu()[live], state[live], rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,D,Dv", [(4, 32, 32), (3, 48, 20), (1, 256, 64)])
+def test_tied_gate_recurrence(dtype, H, D, Dv):
+    torch.manual_seed(5)
+    gb, cb, _ = make_batch("cuda")
+    N = gb.num_tokens
+    q, f, v = torch.randn(N, H, D).to(dtype), torch.randn(N, H, D).to(dtype), torch.randn(N, H, Dv).to(dtype)
+    fb, low = torch.randn(H * D), torch.rand(H * D)
+    state = torch.randn(6, H, D, Dv)
+    sg = state.cuda()
+    out = linear_recurrence.tied_gate_recurrence(q.cuda(), f.cuda(), v.cuda(), fb.cuda(), low.cuda(), sg, gb)
+    ref = linear_recurrence.tied_gate_recurrence_ref(q, f, v, fb, low, state, cb)
+    torch.testing.assert_close(out.cpu(), ref, rtol=2e-4, atol=2e-4)
+    live = sorted(gb.slots_host)
+    torch.testing.assert_close(sg.cpu()[live], state[live], rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv,window,keep", [(4, 2, 32, 32, 9, 3), (6, 3, 24, 40, 0, 0), (2, 2, 64, 16, 70, 0),
+                                                  (4, 1, 16, 130, 5, 30)])
+def test_paged_attention(dtype, H, G, D, Dv, window, keep):
+    torch.manual_seed(6)
+    gb, cb, pages = make_batch("cuda")
+    N = gb.num_tokens
+    kpool, vpool = torch.randn(pages, 16, G, D).to(dtype), torch.randn(pages, 16, G, Dv).to(dtype)
+    kg, vg = kpool.cuda(), vpool.cuda()
+    q, k, v = torch.randn(N, H, D).to(dtype), torch.randn(N, G, D).to(dtype), torch.randn(N, G, Dv).to(dtype)
+    gate = torch.randn(N, H).to(dtype)
+    slopes = paged_attention.distance_slopes(H)
+    paged_attention.paged_kv_write(k.cuda(), v.cuda(), kg, vg, gb)
+    paged_attention.paged_kv_write(k, v, kpool, vpool, cb)
+    torch.testing.assert_close(kg.cpu(), kpool)
+    out = paged_attention.paged_attention(q.cuda(), kg, vg, gb, 0.2, window, keep, slopes.cuda(), gate.cuda())
+    ref = paged_attention.paged_attention_ref(q, kpool, vpool, cb, 0.2, window, keep, slopes, gate)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **(tol(dtype) if dtype == torch.bfloat16
+                                                                 else dict(rtol=1e-4, atol=1e-4)))
+
+
+def test_activations():
+    x = torch.randn(1000)
+    torch.testing.assert_close(relu_squared(x.cuda()).cpu(), torch.relu(x).square())
+    xb = x.bfloat16()
+    torch.testing.assert_close(relu_squared(xb.cuda()).cpu(), torch.relu(xb).square())
+    torch.testing.assert_close(softcap(x.cuda() * 20, 15.0).cpu(), 15.0 * torch.tanh(x * 20 / 15.0), rtol=1e-5, atol=1e-5)
