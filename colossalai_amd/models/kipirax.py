@@ -318,6 +318,8 @@ class KipiraxForCausalLM(nn.Module):
                 put(layer.norm2, get(p + "norm2"))
                 put(layer.mlp.up.weight, get(p + "mlp.up"))
                 put(layer.mlp.down.weight, get(p + "mlp.down"))
+            else:
+                used.add(p + "norm2")  # a layer without a feed-forward may still carry its unused norm weight
             if layer.kind == "parallel":
                 a, b = p + "mix.left.", p + "mix.right."
                 pack(m.in_proj, {"lq": a + "q", "lk": a + "k", "lv": a + "v", "lg": a + "g",
