@@ -24,7 +24,8 @@ at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, 
                                 at::Tensor state, at::Tensor cu, at::Tensor start, at::Tensor slots);
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
-                           int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate);
+                           int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
+                           int64_t num_tiles);
 
 }  // namespace serving
 }  // namespace cai

@@ -2,12 +2,12 @@
 //
 // Each head keeps S [D, Dv] per state slot. Columns of S (value channels) are
 // independent in both update rules, so a value channel is owned by P adjacent
-// lanes that split the D rows between them (16 rows per lane, in registers);
-// the two dot products per token are reduced across those P lanes. A wave
-// walks its sequence's new tokens in order, so prompt portions and single
-// decode tokens are the same code, and the state only touches memory at the
-// start and the end of a portion: cutting a prompt differently cannot change
-// a result.
+// lanes that split the D rows between them (8 or 16 rows per lane, in
+// registers); the two dot products per token are reduced across those P lanes.
+// A wave walks its sequence's new tokens in order, so prompt portions and
+// single decode tokens are the same code, and the state only touches memory at
+// the start and the end of a portion: cutting a prompt differently cannot
+// change a result.
 //
 //   delta: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
 //   tied : S <- diag(f) S + (1 - f) v^T;                          o = S^T q
@@ -20,7 +20,6 @@
 namespace cai {
 namespace serving {
 
-constexpr int DPL = 16;  // rows of S per lane
 
 // ------------------------------------------------------------------ prologue
 // One block per token. q/k [N, G, D] row-strided; dt [N, H*D] row-strided.
@@ -68,43 +67,55 @@ __global__ __launch_bounds__(256) void tied_prepare_kernel(
 }
 
 // ---------------------------------------------------------------------- scan
-DEV_INLINE void load_rows(float* dst, const float* base, int d0, int D, bool vec, float fill) {
-  if (vec && d0 + DPL <= D) {
-#pragma unroll
-    for (int j = 0; j < DPL; j += 4) {
-      const float4v t = *reinterpret_cast<const float4v*>(base + d0 + j);
-      dst[j] = t[0]; dst[j + 1] = t[1]; dst[j + 2] = t[2]; dst[j + 3] = t[3];
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < DPL; ++j) dst[j] = (d0 + j < D) ? base[d0 + j] : fill;
-  }
+// Sum over the P adjacent lanes that share a value channel, on the DPP path
+// (no LDS traffic): xor 1 and 2 inside a quad, then the half-row and row
+// mirrors pair up quads and octets whose lanes already hold equal sums.
+template <int CTRL>
+DEV_INLINE float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+  return v + __builtin_bit_cast(float, moved);
 }
 
 template <int P>
 DEV_INLINE float reduce_p(float v) {
-#pragma unroll
-  for (int off = 1; off < P; off <<= 1) v += __shfl_xor(v, off);
+  if (P >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  if (P >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  if (P >= 8) v = dpp_add<0x141>(v);  // row_half_mirror
+  if (P >= 16) v = dpp_add<0x140>(v); // row_mirror
   return v;
 }
 
-// grid (ceil(Dv / (64 / P)), H, B), one wave per block.
+// grid (ceil(Dv / (4 * 64 / P)), H, B), four waves per block; lane = (value channel, row slice p).
 // q, k: [N, Hq, D] float (Hq = H / rep); gate: [N, H, D] float (decay g or forget f).
-template <int P, bool DELTA, typename TV>
-__global__ __launch_bounds__(64) void matrix_state_scan_kernel(
+// The block stages CT tokens' operand rows of its head in LDS (double-buffered: the next chunk's
+// global loads are in flight while this chunk's tokens are stepped through).
+template <int P, int DPL, bool DELTA, typename TV>
+__global__ __launch_bounds__(256) void matrix_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ gate,
     const float* __restrict__ beta, const TV* __restrict__ v, long vs, float* __restrict__ state, long ss,
     const int* __restrict__ cu, const int* __restrict__ start, const int* __restrict__ slots, int H, int rep, int D,
     int Dv) {
+  constexpr int Dp = P * DPL;                 // padded key size
+  constexpr int CT = Dp > 128 ? 8 : 16;       // tokens per staged chunk
+  constexpr int NOPS = DELTA ? 3 : 2;         // q, (k,) gate
+  constexpr int CPB = 4 * 64 / P;             // value channels per block
+  constexpr int OPF = CT * NOPS * Dp;         // operand floats per chunk
+  constexpr int R_OP = (OPF + 255) / 256;
+  constexpr int R_V = (CT * CPB + 255) / 256;
+  extern __shared__ __align__(16) float lds[];
+  float* ops_buf = lds;                       // [2][CT][NOPS][Dp]
+  float* v_buf = lds + 2 * OPF;               // [2][CT][CPB]
+  float* b_buf = v_buf + 2 * CT * CPB;        // [2][CT]
+
   const int b = blockIdx.z, h = blockIdx.y;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int p = lane % P;
-  const int c = blockIdx.x * (64 / P) + lane / P;
+  const int cl = wid * (64 / P) + lane / P;   // channel inside the block
+  const int c = blockIdx.x * CPB + cl;
   const bool live = c < Dv;
   const int cc = live ? c : Dv - 1;
   const int d0 = p * DPL;
   const int Hq = H / rep, hq = h / rep;
-  const bool vec = (D % 4) == 0;
   const int t0 = cu[b], t1 = cu[b + 1];
   float* Sg = state + (long)slots[b] * ss + (long)h * D * Dv;
 
@@ -113,50 +124,95 @@ __global__ __launch_bounds__(64) void matrix_state_scan_kernel(
 #pragma unroll
   for (int j = 0; j < DPL; ++j) S[j] = (!fresh && d0 + j < D) ? Sg[(long)(d0 + j) * Dv + cc] : 0.0f;
 
-  float qn[DPL], kn[DPL], gn[DPL], vn, bn = 0.0f;
-  // operands of the first token
-  load_rows(qn, q + ((long)t0 * Hq + hq) * D, d0, D, vec, 0.0f);
-  if (DELTA) load_rows(kn, k + ((long)t0 * Hq + hq) * D, d0, D, vec, 0.0f);
-  load_rows(gn, gate + ((long)t0 * H + h) * D, d0, D, vec, 1.0f);
-  vn = ldf(v + (long)t0 * vs + (long)h * Dv + cc);
-  if (DELTA) bn = beta[(long)t0 * H + h];
+  float r_op[R_OP], r_v[R_V], r_b = 0.0f;
+  auto fetch = [&](int tb) {  // chunk starting at token tb -> registers
+#pragma unroll
+    for (int r = 0; r < R_OP; ++r) {
+      const int i = tid + 256 * r;
+      const int tok = i / (NOPS * Dp), op = (i / Dp) % NOPS, d = i % Dp;
+      const int t = tb + tok;
+      float val = (op == NOPS - 1) ? 1.0f : 0.0f;
+      if (i < OPF && t < t1 && d < D) {
+        if (op == NOPS - 1) val = gate[((long)t * H + h) * D + d];
+        else if (op == 0) val = q[((long)t * Hq + hq) * D + d];
+        else val = k[((long)t * Hq + hq) * D + d];
+      }
+      r_op[r] = val;
+    }
+#pragma unroll
+    for (int r = 0; r < R_V; ++r) {
+      const int i = tid + 256 * r;
+      const int tok = i / CPB, ch = min((int)(blockIdx.x * CPB + i % CPB), Dv - 1);
+      const int t = tb + tok;
+      r_v[r] = (i < CT * CPB && t < t1) ? ldf(v + (long)t * vs + (long)h * Dv + ch) : 0.0f;
+    }
+    if (DELTA) r_b = (tid < CT && tb + tid < t1) ? beta[(long)(tb + tid) * H + h] : 0.0f;
+  };
+  auto stash = [&](int buf) {  // registers -> LDS buffer
+#pragma unroll
+    for (int r = 0; r < R_OP; ++r) {
+      const int i = tid + 256 * r;
+      if (i < OPF) ops_buf[buf * OPF + i] = r_op[r];
+    }
+#pragma unroll
+    for (int r = 0; r < R_V; ++r) {
+      const int i = tid + 256 * r;
+      if (i < CT * CPB) v_buf[buf * CT * CPB + i] = r_v[r];
+    }
+    if (DELTA && tid < CT) b_buf[buf * CT + tid] = r_b;
+  };
 
-  for (int t = t0; t < t1; ++t) {
-    float qc[DPL], kc[DPL], gc[DPL];
+  fetch(t0);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int tb = t0; tb < t1; tb += CT, buf ^= 1) {
+    const bool more = tb + CT < t1;
+    if (more) fetch(tb + CT);
+    const int cnt = min(CT, t1 - tb);
+    for (int tt = 0; tt < cnt; ++tt) {
+      const float* row = ops_buf + buf * OPF + tt * NOPS * Dp + d0;
+      float qc[DPL], kc[DPL], gc[DPL];
 #pragma unroll
-    for (int j = 0; j < DPL; ++j) { qc[j] = qn[j]; gc[j] = gn[j]; if (DELTA) kc[j] = kn[j]; }
-    const float vc = vn, bc = bn;
-    if (t + 1 < t1) {  // fetch the next token's operands while this one computes
-      load_rows(qn, q + ((long)(t + 1) * Hq + hq) * D, d0, D, vec, 0.0f);
-      if (DELTA) load_rows(kn, k + ((long)(t + 1) * Hq + hq) * D, d0, D, vec, 0.0f);
-      load_rows(gn, gate + ((long)(t + 1) * H + h) * D, d0, D, vec, 1.0f);
-      vn = ldf(v + (long)(t + 1) * vs + (long)h * Dv + cc);
-      if (DELTA) bn = beta[(long)(t + 1) * H + h];
+      for (int j = 0; j < DPL; j += 4) {
+        const float4v a = *reinterpret_cast<const float4v*>(row + j);
+        qc[j] = a[0]; qc[j + 1] = a[1]; qc[j + 2] = a[2]; qc[j + 3] = a[3];
+        if (DELTA) {
+          const float4v kk = *reinterpret_cast<const float4v*>(row + Dp + j);
+          kc[j] = kk[0]; kc[j + 1] = kk[1]; kc[j + 2] = kk[2]; kc[j + 3] = kk[3];
+        }
+        const float4v gg = *reinterpret_cast<const float4v*>(row + (NOPS - 1) * Dp + j);
+        gc[j] = gg[0]; gc[j + 1] = gg[1]; gc[j + 2] = gg[2]; gc[j + 3] = gg[3];
+      }
+      const float vc = v_buf[buf * CT * CPB + tt * CPB + cl];
+      float o = 0.0f;
+      if (DELTA) {
+        const float bc = b_buf[buf * CT + tt];
+        float dot = 0.0f;
+#pragma unroll
+        for (int j = 0; j < DPL; ++j) {
+          S[j] *= gc[j];
+          dot += S[j] * kc[j];
+        }
+        dot = reduce_p<P>(dot);
+        const float u = bc * (vc - dot);
+#pragma unroll
+        for (int j = 0; j < DPL; ++j) {
+          S[j] += kc[j] * u;
+          o += S[j] * qc[j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < DPL; ++j) {
+          S[j] = gc[j] * S[j] + (1.0f - gc[j]) * vc;
+          o += S[j] * qc[j];
+        }
+      }
+      o = reduce_p<P>(o);
+      if (p == 0 && live) out[((long)(tb + tt) * H + h) * Dv + c] = o;
     }
-    float o = 0.0f;
-    if (DELTA) {
-      float dot = 0.0f;
-#pragma unroll
-      for (int j = 0; j < DPL; ++j) {
-        S[j] *= gc[j];
-        dot += S[j] * kc[j];
-      }
-      dot = reduce_p<P>(dot);
-      const float u = bc * (vc - dot);
-#pragma unroll
-      for (int j = 0; j < DPL; ++j) {
-        S[j] += kc[j] * u;
-        o += S[j] * qc[j];
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < DPL; ++j) {
-        S[j] = gc[j] * S[j] + (1.0f - gc[j]) * vc;
-        o += S[j] * qc[j];
-      }
-    }
-    o = reduce_p<P>(o);
-    if (p == 0 && live) out[((long)t * H + h) * Dv + c] = o;
+    if (more) stash(buf ^ 1);
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -169,18 +225,22 @@ template <bool DELTA, typename TV>
 static void launch_scan(float* out, const float* q, const float* k, const float* gate, const float* beta, const TV* v,
                         long vs, float* state, long ss, const int* cu, const int* start, const int* slots, int B,
                         int H, int rep, int D, int Dv) {
+  TORCH_CHECK(D <= 256, "key size above 256 is not supported by the recurrence kernel");
+  const int dpl = D > 128 ? 16 : 8;
   int P = 1;
-  while (P * DPL < D) P <<= 1;
-  TORCH_CHECK(P <= 16, "key size above 256 is not supported by the recurrence kernel");
-  const dim3 grid((unsigned)((Dv + 64 / P - 1) / (64 / P)), (unsigned)H, (unsigned)B);
-#define SCAN_CASE(PP)                                                                                              \
-  case PP:                                                                                                         \
-    hipLaunchKernelGGL((matrix_state_scan_kernel<PP, DELTA, TV>), grid, dim3(64), 0, stream(), out, q, k, gate,    \
-                       beta, v, vs, state, ss, cu, start, slots, H, rep, D, Dv);                                   \
-    break;
-  switch (P) {
-    SCAN_CASE(1) SCAN_CASE(2) SCAN_CASE(4) SCAN_CASE(8) SCAN_CASE(16)
-  }
+  while (P * dpl < D) P <<= 1;
+  const int cpb = 4 * 64 / P, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
+  const dim3 grid((unsigned)((Dv + cpb - 1) / cpb), (unsigned)H, (unsigned)B);
+  const size_t smem = (size_t)(2 * ct * nops * Dp + 2 * ct * cpb + 2 * ct) * sizeof(float);
+#define SCAN_CASE(PP, DD)                                                                                          \
+  hipLaunchKernelGGL((matrix_state_scan_kernel<PP, DD, DELTA, TV>), grid, dim3(256), smem, stream(), out, q, k,   \
+                     gate, beta, v, vs, state, ss, cu, start, slots, H, rep, D, Dv)
+  if (dpl == 16) SCAN_CASE(16, 16);
+  else if (P == 1) SCAN_CASE(1, 8);
+  else if (P == 2) SCAN_CASE(2, 8);
+  else if (P == 4) SCAN_CASE(4, 8);
+  else if (P == 8) SCAN_CASE(8, 8);
+  else SCAN_CASE(16, 8);
 #undef SCAN_CASE
   HIP_CHECK_LAST();
 }

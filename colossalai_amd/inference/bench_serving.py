@@ -1,0 +1,131 @@
+"""Serving throughput of the hybrid (paged window attention + recurrent state)
+model next to a Llama of equal width, depth and parameter budget, both through
+``ContinuousBatchEngine``: prefill tokens/s of one long prompt and decode
+tokens/s of a batch of running sequences. Random weights, synthetic tokens.
+"""
+
+import json
+import time
+from typing import Dict, List
+
+import torch
+
+from ..models import KipiraxConfig, KipiraxForCausalLM, LlamaConfig, LlamaForCausalLM
+from .config import InferenceConfig
+from .paged_engine import ContinuousBatchEngine
+
+__all__ = ["SIZES", "hybrid_config", "llama_config", "run_serving_comparison"]
+
+# width, layers, heads, kv_heads, head size, vocab
+SIZES = {
+    "w2048": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, vocab=32000),
+    "w4096": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, vocab=32000),
+}
+
+
+def hybrid_config(s: dict, max_positions: int, window: int = 1024, keep_first: int = 4) -> KipiraxConfig:
+    W, H, G, D = s["width"], s["heads"], s["kv_heads"], s["dim"]
+    left = dict(dim=D, heads=H, kv_heads=G, vdim=D, scale=D ** -0.5, mask=dict(size=window, keep_first=keep_first))
+    right = dict(dim=D // 2, heads=H // 2, vdim=D)
+    delta = dict(conv=4, dim=D, heads=H, kv_heads=H, vdim=D, decay_rank=W // 16, gate_rank=W // 16)
+    layers = []
+    for i in range(s["layers"]):
+        mixer = dict(left=left, right=right) if i % 2 == 0 else delta
+        layers.append(dict(type="parallel" if i % 2 == 0 else "channel_delta", mixer=mixer,
+                           mlp=dict(kind="dense", ff=4 * W)))
+    return KipiraxConfig(vocab=s["vocab"], width=W, max_positions=max_positions, layers=layers, norm_eps=1e-6,
+                         norm_groups=4, logit_softcap=30.0)
+
+
+def llama_config(s: dict, max_positions: int) -> LlamaConfig:
+    # gate/up/down of 8/3 W carry the parameters of the hybrid's up/down of 4 W
+    inter = (8 * s["width"] // 3 + 255) // 256 * 256
+    return LlamaConfig(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=inter,
+                       num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
+                       num_key_value_heads=s["kv_heads"], max_position_embeddings=max_positions)
+
+
+def _random(model: torch.nn.Module, dtype) -> torch.nn.Module:
+    model = model.to(device="cuda")
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() >= 2:
+                p.data = p.data.to(dtype)
+                p.normal_(0, 0.02)
+    return model.eval()
+
+
+def _timed(fn, repeats: int) -> float:
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / repeats
+
+
+def _hybrid_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
+    page = 64
+    cfg = hybrid_config(s, max_positions=max(prompt, context + steps + 8) + 8)
+    model = _random(KipiraxForCausalLM(cfg), torch.bfloat16)
+    blocks = max(prompt, batch * (context + steps + page)) // page + batch + 2
+    eng = ContinuousBatchEngine(model, InferenceConfig(max_batch_size=batch + 1), num_blocks=blocks, block_size=page)
+    toks = torch.randint(0, cfg.vocab, (prompt,)).tolist()
+
+    def prefill():
+        eng.run_ragged([("p", toks, [prompt - 1])])
+        eng.close_sequence("p")
+
+    t_prefill = _timed(prefill, 3)
+    ctx = torch.randint(0, cfg.vocab, (batch, context)).tolist()
+    eng.run_ragged([(i, ctx[i], [context - 1]) for i in range(batch)])
+
+    def decode():
+        eng.run_ragged([(i, [1], [0]) for i in range(batch)])
+
+    t_decode = _timed(decode, steps)
+    params = sum(p.numel() for p in model.parameters())
+    del eng, model
+    torch.cuda.empty_cache()
+    return dict(prefill_tok_s=prompt / t_prefill, decode_tok_s=batch / t_decode, decode_ms=t_decode * 1e3, params=params)
+
+
+def _llama_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
+    from .config import GenerationConfig
+
+    cfg = llama_config(s, max_positions=max(prompt, context + steps + 8) + 8)
+    model = _random(LlamaForCausalLM(cfg), torch.bfloat16).to(torch.bfloat16)
+    icfg = InferenceConfig(max_batch_size=batch, max_input_len=max(prompt, context), max_output_len=steps + 8)
+    eng = ContinuousBatchEngine(model, icfg, block_size=16)
+    toks = torch.randint(0, cfg.vocab_size, (1, prompt), device="cuda")
+    lens = torch.tensor([prompt], device="cuda", dtype=torch.int32)
+    pos = torch.arange(prompt, device="cuda").int()
+
+    @torch.inference_mode()
+    def prefill():
+        eng.kv.allocate(-1, prompt)
+        eng._forward(toks, pos, [-1], None, lens, True)
+        eng.kv.free(-1)
+
+    t_prefill = _timed(prefill, 3)
+    eng._gen = GenerationConfig(max_new_tokens=steps + 4)
+    for row in torch.randint(0, cfg.vocab_size, (batch, context)).tolist():
+        eng.add_request(row, steps + 4)
+    eng.step()  # prefill of the batch + first decode
+    t_decode = _timed(eng.step, steps)
+    params = sum(p.numel() for p in model.parameters())
+    del eng, model
+    torch.cuda.empty_cache()
+    return dict(prefill_tok_s=prompt / t_prefill, decode_tok_s=batch / t_decode, decode_ms=t_decode * 1e3, params=params)
+
+
+def run_serving_comparison(sizes: List[str], prompt: int = 4096, batch: int = 16, context: int = 1024,
+                           steps: int = 32) -> dict:
+    out = {}
+    for name in sizes:
+        s = SIZES[name]
+        out[name] = {"hybrid": _hybrid_numbers(s, prompt, batch, context, steps),
+                     "llama": _llama_numbers(s, prompt, batch, context, steps),
+                     "shape": dict(s, prompt=prompt, batch=batch, context=context)}
+    return out
