@@ -82,5 +82,56 @@ def check(installation):
     print(f"colossalai_amd: {colossalai_amd.__version__}")
 
 
+@cli.command()
+@click.option("--model", "model_dir", required=True, help="folder with config.json and model.safetensors")
+@click.option("--prompt-ids", required=True, help="comma-separated token ids; ';' between prompts")
+@click.option("--max-new-tokens", type=int, default=32)
+@click.option("--dtype", type=click.Choice(["bfloat16", "float32"]), default="bfloat16")
+@click.option("--temperature", type=float, default=0.0, help="0 = greedy")
+@click.option("--top-k", type=int, default=0)
+@click.option("--top-p", type=float, default=1.0)
+@click.option("--max-batch-size", type=int, default=8)
+@click.option("--max-step-tokens", type=int, default=2048, help="token budget of one engine step (chunked prefill)")
+def generate(model_dir, prompt_ids, max_new_tokens, dtype, temperature, top_k, top_p, max_batch_size, max_step_tokens):
+    """Generate from token ids with any registered model (class chosen by config.json)."""
+    import json
+
+    import torch
+
+    from colossalai_amd.inference import ContinuousBatchEngine, GenerationConfig, InferenceConfig
+    from colossalai_amd.models import load_pretrained
+
+    td = torch.float32 if dtype == "float32" else torch.bfloat16
+    device = "cuda" if torch.cuda.is_available() else "cpu"
+    model = load_pretrained(model_dir, dtype=td, device=device)
+    prompts = [[int(t) for t in part.split(",") if t.strip()] for part in prompt_ids.split(";") if part.strip()]
+    longest = max(len(p) for p in prompts)
+    engine = ContinuousBatchEngine(
+        model, InferenceConfig(max_batch_size=max_batch_size, max_input_len=longest, max_output_len=max_new_tokens, dtype=td),
+        max_step_tokens=max_step_tokens)
+    gen = GenerationConfig(max_new_tokens=max_new_tokens, do_sample=temperature > 0, temperature=max(temperature, 1e-5),
+                           top_k=top_k, top_p=top_p)
+    for p, out in zip(prompts, engine.generate(prompts, gen)):
+        print(json.dumps({"prompt_ids": p, "output_ids": out[len(p):]}))
+
+
+@cli.command(context_settings=dict(ignore_unknown_options=True))
+@click.argument("args", nargs=-1, type=click.UNPROCESSED)
+def replay(args):
+    """Replay a token trace through the serving engine and write logits (see `replay --help-trace`;
+    arguments as bin/trace_run: --model DIR --dtype T --out DIR --max-tokens N, steps on stdin)."""
+    from colossalai_amd.inference.trace_replay import main as replay_main
+
+    sys.exit(replay_main(["--help"] if "--help-trace" in args else list(args)))
+
+
+@cli.command()
+def models():
+    """List the architectures the model registry can load."""
+    from colossalai_amd.models import registered_models
+
+    print("\n".join(registered_models()))
+
+
 if __name__ == "__main__":
     cli()
