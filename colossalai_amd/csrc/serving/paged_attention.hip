@@ -15,142 +15,213 @@
 namespace cai {
 namespace serving {
 
-constexpr int MAX_VD_PER_LANE = 4;  // value size up to 256
-constexpr int ATT_WAVES = 4;        // waves of a block: they split the keys of one (token, head)
+constexpr int ATT_WAVES = 8;  // waves of a block: they split the key blocks of one (token, kv head)
+constexpr int RC = 4;         // query heads of the kv head's group handled together by a block
 
-DEV_INLINE float dot_row(const float* kr, const float* qs, int D, bool vec) {
-  float dot = 0.0f;
-  if (vec) {
-    for (int d = 0; d < D; d += 4) {
-      const float4v kv = *reinterpret_cast<const float4v*>(kr + d);
-      const float4v qv = *reinterpret_cast<const float4v*>(qs + d);
-      dot += kv[0] * qv[0] + kv[1] * qv[1] + kv[2] * qv[2] + kv[3] * qv[3];
-    }
-  } else {
-    for (int d = 0; d < D; ++d) dot += qs[d] * kr[d];
-  }
-  return dot;
+template <int CTRL>
+DEV_INLINE float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+  return v + __builtin_bit_cast(float, moved);
 }
+// sum over the 8 adjacent lanes that share a key (quad xor 1, quad xor 2, half-row mirror)
+DEV_INLINE float reduce8(float v) { return dpp_add<0x141>(dpp_add<0x4E>(dpp_add<0xB1>(v))); }
 
-DEV_INLINE float dot_row(const bf16s* kr, const float* qs, int D, bool vec) {
-  float dot = 0.0f;
-  if (vec) {
-    for (int d = 0; d < D; d += 8) {
-      const short8 kv = *reinterpret_cast<const short8*>(kr + d);
-      const float4v qa = *reinterpret_cast<const float4v*>(qs + d);
-      const float4v qb = *reinterpret_cast<const float4v*>(qs + d + 4);
-      dot += bf2f((bf16s)kv[0]) * qa[0] + bf2f((bf16s)kv[1]) * qa[1] + bf2f((bf16s)kv[2]) * qa[2] +
-             bf2f((bf16s)kv[3]) * qa[3] + bf2f((bf16s)kv[4]) * qb[0] + bf2f((bf16s)kv[5]) * qb[1] +
-             bf2f((bf16s)kv[6]) * qb[2] + bf2f((bf16s)kv[7]) * qb[3];
-    }
-  } else {
-    for (int d = 0; d < D; ++d) dot += qs[d] * bf2f(kr[d]);
-  }
-  return dot;
+// 8 consecutive elements of a key row as floats
+DEV_INLINE void load8(const float* p, float* o) {
+  const float4v a = *reinterpret_cast<const float4v*>(p), b = *reinterpret_cast<const float4v*>(p + 4);
+  o[0] = a[0]; o[1] = a[1]; o[2] = a[2]; o[3] = a[3]; o[4] = b[0]; o[5] = b[1]; o[6] = b[2]; o[7] = b[3];
+}
+DEV_INLINE void load8(const bf16s* p, float* o) {
+  const short8 a = *reinterpret_cast<const short8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = bf2f((bf16s)a[e]);
+}
+// two consecutive value channels
+DEV_INLINE void load2(const float* p, float& a, float& b) {
+  const float2v t = *reinterpret_cast<const float2v*>(p);
+  a = t[0]; b = t[1];
+}
+DEV_INLINE void load2(const bf16s* p, float& a, float& b) {
+  const unsigned int t = *reinterpret_cast<const unsigned int*>(p);
+  a = bf2f((bf16s)(t & 0xffffu)); b = bf2f((bf16s)(t >> 16));
 }
 
 // Scalar kernel (decode tokens, float32 serving, shapes the MFMA kernel does not take).
-// One block per (token, head); its four waves take every fourth 64-key block and merge
-// their partial softmax states through LDS.
+// One block per (token, kv head, group of up to RC query heads of that kv head): keys and
+// values are read once for the whole group. The block's waves take every ATT_WAVES-th block
+// of 64 keys and merge their partial softmax states through LDS at the end.
+// Scores: 8 adjacent lanes share a key, each takes a contiguous slice of the head size
+// (16-byte loads, few cache lines per instruction) and the slices are summed on the DPP path.
+// Values: lane = a pair of value channels, the block's weights and pool rows come from LDS.
 template <typename T>
 __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, const float* __restrict__ slopes, const T* __restrict__ gate, long gate_stride,
-    int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec) {
+    int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec, int vvec) {
   extern __shared__ __align__(16) float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int Dp = (D + 3) & ~3;
-  float* qs = lds;                                   // [Dp] query
-  float* pw = lds + Dp + wid * 128;                  // [64] weights of this wave's key block
-  int* prow = reinterpret_cast<int*>(pw + 64);       // [64] pool rows of the block
-  float* part = lds + Dp + ATT_WAVES * 128;          // [waves][2 + Dv] partial states
-  const long n = blockIdx.x / H;
-  const int h = (int)(blockIdx.x % H);
-  const int g = h / (H / G);
+  const int Dp = (D + 7) & ~7;
+  const int R = H / G, chunks = (R + RC - 1) / RC;
+  float* qs = lds;                                        // [RC][Dp] queries
+  float* pw = lds + RC * Dp + wid * (RC * 64 + 64);       // [RC][64] scores, then weights, of this wave's key block
+  int* prow = reinterpret_cast<int*>(pw + RC * 64);       // [64] pool rows of the block
+  float* part = lds + RC * Dp + ATT_WAVES * (RC * 64 + 64);  // [waves][RC][2 + Dv] partial states
+  const long n = blockIdx.x / (G * chunks);
+  const int g = (int)(blockIdx.x / chunks) % G;
+  const int h0 = g * R + (int)(blockIdx.x % chunks) * RC;  // first query head of this block
+  const int nh = min(RC, g * R + R - h0);
   const int b = tok_seq[n];
   const int pos = positions[n];
   const int* bt = block_tables + (long)b * bt_stride;
   const int page_mask = (1 << page_shift) - 1;
 
-  for (int i = threadIdx.x; i < D; i += blockDim.x) qs[i] = ldf(q + n * q_stride + (long)h * D + i);
+  for (int i = threadIdx.x; i < RC * Dp; i += blockDim.x) {
+    const int r = i / Dp, d = i % Dp;
+    qs[i] = (r < nh && d < D) ? ldf(q + n * q_stride + (long)(h0 + r) * D + d) : 0.0f;
+  }
   __syncthreads();
-  const float slope = slopes != nullptr ? slopes[h] : 0.0f;
+  float slope[RC];
+#pragma unroll
+  for (int r = 0; r < RC; ++r) slope[r] = (slopes != nullptr && r < nh) ? slopes[h0 + r] : 0.0f;
 
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int n_keep = window > 0 ? min(keep_first, lo) : 0;
   const int total = n_keep + (pos - lo + 1);
+  const int part8 = lane & 7, ksub = lane >> 3;
+  const int DS = (((D + 7) >> 3) + 7) & ~7;  // slice of the head size per lane, a multiple of 8
+  const int d_lo = part8 * DS, d_hi = min(D, d_lo + DS);
 
-  float m = -INFINITY, l = 0.0f;
-  float acc[MAX_VD_PER_LANE];
+  float m[RC], l[RC], acc[RC][4];
 #pragma unroll
-  for (int i = 0; i < MAX_VD_PER_LANE; ++i) acc[i] = 0.0f;
+  for (int r = 0; r < RC; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
+  }
 
   for (int base = wid * 64; base < total; base += 64 * ATT_WAVES) {
-    const int idx = base + lane;
-    const bool valid = idx < total;
-    float s = -INFINITY;
-    int row = 0;
-    if (valid) {
-      const int j = idx < n_keep ? idx : lo + (idx - n_keep);
-      row = (bt[j >> page_shift] << page_shift) + (j & page_mask);
-      s = dot_row(kpool + ((long)row * G + g) * D, qs, D, kvec != 0) * scale - slope * (float)(pos - j);
+#pragma unroll 2
+    for (int sub = 0; sub < 8; ++sub) {
+      const int idx = base + sub * 8 + ksub;
+      const bool valid = idx < total;
+      const int j = valid ? (idx < n_keep ? idx : lo + (idx - n_keep)) : pos;
+      const int row = (bt[j >> page_shift] << page_shift) + (j & page_mask);
+      float dots[RC];
+#pragma unroll
+      for (int r = 0; r < RC; ++r) dots[r] = 0.0f;
+      const T* kr = kpool + ((long)row * G + g) * D;
+      if (kvec) {
+        for (int d = d_lo; d < d_hi; d += 8) {
+          float kv[8];
+          load8(kr + d, kv);
+#pragma unroll
+          for (int r = 0; r < RC; ++r) {
+            const float4v qa = *reinterpret_cast<const float4v*>(qs + r * Dp + d);
+            const float4v qb = *reinterpret_cast<const float4v*>(qs + r * Dp + d + 4);
+            dots[r] += kv[0] * qa[0] + kv[1] * qa[1] + kv[2] * qa[2] + kv[3] * qa[3] + kv[4] * qb[0] + kv[5] * qb[1] +
+                       kv[6] * qb[2] + kv[7] * qb[3];
+          }
+        }
+      } else {
+        for (int d = d_lo; d < d_hi; ++d) {
+          const float kv = ldf(kr + d);
+#pragma unroll
+          for (int r = 0; r < RC; ++r) dots[r] += kv * qs[r * Dp + d];
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < RC; ++r) dots[r] = reduce8(dots[r]);
+      if (part8 == 0) {
+#pragma unroll
+        for (int r = 0; r < RC; ++r)
+          pw[r * 64 + sub * 8 + ksub] = valid ? dots[r] * scale - slope[r] * (float)(pos - j) : -INFINITY;
+        prow[sub * 8 + ksub] = row;
+      }
     }
-    const float m_new = fmaxf(m, wave_reduce_max(s));  // a block holds at least one valid key
-    const float w = valid ? expf(s - m_new) : 0.0f;
-    const float corr = expf(m - m_new);  // m = -inf on the first block: exp(-inf) = 0
-    l = l * corr + wave_reduce_sum(w);
-    m = m_new;
-    pw[lane] = w;
-    prow[lane] = row;
     // the wave is its own producer and consumer of pw/prow: wait for its LDS writes
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-    const int cnt = min(64, total - base);
+    float corr[RC];
 #pragma unroll
-    for (int i = 0; i < MAX_VD_PER_LANE; ++i) {
-      const int dv = lane + 64 * i;
-      if (dv < Dv) {
-        float a = acc[i] * corr;
-        for (int jj = 0; jj < cnt; ++jj) a += pw[jj] * ldf(vpool + ((long)prow[jj] * G + g) * Dv + dv);
-        acc[i] = a;
+    for (int r = 0; r < RC; ++r) {
+      const float s = pw[r * 64 + lane];
+      const float m_new = fmaxf(m[r], wave_reduce_max(s));  // a block holds at least one visible key
+      const float w = expf(s - m_new);                      // exp(-inf) = 0 for the block's empty places
+      corr[r] = expf(m[r] - m_new);                         // m = -inf before the first block: 0
+      l[r] = l[r] * corr[r] + wave_reduce_sum(w);
+      m[r] = m_new;
+      pw[r * 64 + lane] = w;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+#pragma unroll
+    for (int r = 0; r < RC; ++r)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[r][i] *= corr[r];
+    const int cnt = min(64, total - base);
+    const int dva = 2 * lane, dvb = 128 + 2 * lane;
+#pragma unroll 4
+    for (int jj = 0; jj < cnt; ++jj) {
+      const T* vr = vpool + ((long)prow[jj] * G + g) * Dv;
+      float v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
+      if (vvec) {
+        if (dva < Dv) load2(vr + dva, v0, v1);
+        if (dvb < Dv) load2(vr + dvb, v2, v3);
+      } else {
+        if (dva < Dv) v0 = ldf(vr + dva);
+        if (dva + 1 < Dv) v1 = ldf(vr + dva + 1);
+        if (dvb < Dv) v2 = ldf(vr + dvb);
+        if (dvb + 1 < Dv) v3 = ldf(vr + dvb + 1);
+      }
+#pragma unroll
+      for (int r = 0; r < RC; ++r) {
+        const float w = pw[r * 64 + jj];
+        acc[r][0] += w * v0; acc[r][1] += w * v1; acc[r][2] += w * v2; acc[r][3] += w * v3;
       }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
-  float* mine = part + wid * (2 + Dv);
-  if (lane == 0) { mine[0] = m; mine[1] = l; }
+  const int PS = 2 + Dv;
+  float* mine = part + (long)wid * RC * PS;
 #pragma unroll
-  for (int i = 0; i < MAX_VD_PER_LANE; ++i) {
-    const int dv = lane + 64 * i;
-    if (dv < Dv) mine[2 + dv] = acc[i];
+  for (int r = 0; r < RC; ++r) {
+    if (lane == 0) { mine[r * PS] = m[r]; mine[r * PS + 1] = l[r]; }
+    const int dva = 2 * lane, dvb = 128 + 2 * lane;
+    if (dva < Dv) mine[r * PS + 2 + dva] = acc[r][0];
+    if (dva + 1 < Dv) mine[r * PS + 2 + dva + 1] = acc[r][1];
+    if (dvb < Dv) mine[r * PS + 2 + dvb] = acc[r][2];
+    if (dvb + 1 < Dv) mine[r * PS + 2 + dvb + 1] = acc[r][3];
   }
   __syncthreads();
-  float mm = -INFINITY;
-  for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, part[w * (2 + Dv)]);
-  float ll = 0.0f;
-  for (int w = 0; w < ATT_WAVES; ++w) {
-    const float mw = part[w * (2 + Dv)];
-    if (mw != -INFINITY) ll += part[w * (2 + Dv) + 1] * expf(mw - mm);
-  }
-  float scale_out = 1.0f / ll;
-  if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h));
-  for (int dv = threadIdx.x; dv < Dv; dv += blockDim.x) {
-    float o = 0.0f;
+  for (int i = threadIdx.x; i < nh * Dv; i += blockDim.x) {
+    const int r = i / Dv, dv = i % Dv;
+    float mm = -INFINITY;
+    for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, part[(w * RC + r) * PS]);
+    float ll = 0.0f, o = 0.0f;
     for (int w = 0; w < ATT_WAVES; ++w) {
-      const float mw = part[w * (2 + Dv)];
-      if (mw != -INFINITY) o += part[w * (2 + Dv) + 2 + dv] * expf(mw - mm);
+      const float mw = part[(w * RC + r) * PS];
+      if (mw != -INFINITY) {
+        const float f = expf(mw - mm);
+        ll += part[(w * RC + r) * PS + 1] * f;
+        o += part[(w * RC + r) * PS + 2 + dv] * f;
+      }
     }
-    stf(out + (n * H + h) * (long)Dv + dv, o * scale_out);
+    float scale_out = 1.0f / ll;
+    if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h0 + r));
+    stf(out + (n * H + h0 + r) * (long)Dv + dv, o * scale_out);
   }
 }
 
-// MFMA kernel (bfloat16 prompt portions). One wave per (32-token tile of one sequence, head);
-// the four waves of a block take four neighbouring heads of the same tile. All per-token
-// quantities are lane-local because the products are formed transposed:
-//   S^T = K Q^T   (A = key rows, B = query rows: both read along the head size, 16 B a lane)
+// MFMA kernel (bfloat16 prompt portions). One block per (32-token tile of one sequence, kv head,
+// pass); its waves are query heads of that kv head's group, so a key/value tile is fetched once
+// for all of them: 16-byte loads through the page table into LDS, double-buffered (the next
+// tile's loads are in flight while this tile is multiplied). All per-token quantities are
+// lane-local because the products are formed transposed:
+//   S^T = K Q^T   (A = key rows from LDS, B = query rows kept in registers)
 //   O^T = V^T P^T (B = the float32 weights in the C layout they were born in, split into a
 //                  high and a low bfloat16 half so that no weight loses its float32 mantissa
-//                  to the matrix unit; A = values gathered with the same key order)
+//                  to the matrix unit; A = values, stored transposed in LDS in the same key
+//                  order, one 16-byte read per product)
 // so column = token = lane & 31 everywhere: running max, running sum, rescaling and the gate
 // never cross lanes except for one exchange between the two half-waves.
 template <int DS, int VT>
@@ -160,9 +231,18 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const int* __restrict__ start, const float* __restrict__ slopes, const bf16s* __restrict__ gate, long gate_stride,
     int H, int G, int page_shift, float scale, int window, int keep_first) {
   constexpr int D = DS * 16, Dv = VT * 32;
-  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int h = blockIdx.y * 4 + wid;
-  if (h >= H) return;  // waves never synchronise with each other
+  constexpr int KP = D + 8;            // key row pitch in LDS (elements): 16-byte reads of 16 rows hit 64 banks
+  constexpr int VP = 40;               // transposed value row pitch: 32 key slots + 8
+  constexpr int KT = 32 * KP, VTT = Dv * VP;   // elements of one staged tile
+  constexpr int KCH = 32 * D / 8, VCH = 32 * Dv / 8;  // 16-byte chunks of a key / value tile
+  extern __shared__ __align__(16) bf16s tiles[];  // [2][KT + VTT]
+  constexpr int nthreads = 256;  // always four waves: those beyond the group's heads only help staging
+  const int tid = threadIdx.x;
+  const int wid = tid >> 6, lane = tid & 63;
+  const int rep = H / G, g = blockIdx.y;
+  const int hl = blockIdx.z * (nthreads >> 6) + wid;  // head inside the group
+  const bool head_ok = hl < rep;
+  const int h = g * rep + (head_ok ? hl : 0);
   int tile = blockIdx.x, b = 0;
   for (;; ++b) {  // the grid holds exactly sum_b ceil(count_b / 32) tiles
     const int nt = (cu[b + 1] - cu[b] + 31) >> 5;
@@ -178,7 +258,6 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int s0 = start[b];
   const int pos = s0 + my_i;
   const int p0 = s0 + t_off, p1 = s0 + min(t_off + 31, cnt - 1);
-  const int g = h / (H / G);
   const int* bt = block_tables + (long)b * bt_stride;
   const int page_mask = (1 << page_shift) - 1;
   const float slope = slopes != nullptr ? slopes[h] : 0.0f;
@@ -191,7 +270,53 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int wstart = lo_min & ~31;
   const int n_sink = window > 0 ? min(keep_first, wstart) : 0;  // kept keys below the window's first tile
   const int sink_tiles = (n_sink + 31) >> 5;
-  const int tiles = sink_tiles + ((p1 - wstart) >> 5) + 1;
+  const int tiles_n = sink_tiles + ((p1 - wstart) >> 5) + 1;
+
+  // staging: chunk c of a tile = key c / (row chunks), 8 elements starting at 8 * (c % row chunks)
+  constexpr int KR = (KCH + 255) / 256, VR = (VCH + 255) / 256;  // chunks per thread of the 256
+  bf16x8_v rk[KR], rv[VR];
+  auto tile_base = [&](int it) { return it < sink_tiles ? it * 32 : wstart + (it - sink_tiles) * 32; };
+  auto pool_row = [&](int j) {
+    const int jc = min(j, p1);  // keys past the sequence's end are masked; read a row that exists
+    return ((long)bt[jc >> page_shift] << page_shift) + (jc & page_mask);
+  };
+  auto fetch = [&](int it) {
+    const int kbase = tile_base(it);
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+      const int c = tid + nthreads * r;
+      if (c < KCH) rk[r] = ld_g16b(kpool + (pool_row(kbase + c / (D / 8)) * G + g) * D + 8 * (c % (D / 8)));
+    }
+#pragma unroll
+    for (int r = 0; r < VR; ++r) {
+      const int c = tid + nthreads * r;
+      if (c < VCH) rv[r] = ld_g16b(vpool + (pool_row(kbase + c / (Dv / 8)) * G + g) * Dv + 8 * (c % (Dv / 8)));
+    }
+  };
+  auto stash = [&](int buf) {
+    bf16s* ks = tiles + buf * (KT + VTT);
+    bf16s* vt = ks + KT;
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+      const int c = tid + nthreads * r;
+      if (c < KCH) *reinterpret_cast<bf16x8_v*>(ks + (c / (D / 8)) * KP + 8 * (c % (D / 8))) = rk[r];
+    }
+#pragma unroll
+    for (int r = 0; r < VR; ++r) {
+      const int c = tid + nthreads * r;
+      if (c < VCH) {
+        const int kk = c / (Dv / 8), dv0 = 8 * (c % (Dv / 8));
+        // contraction slot of key kk: the order in which the C layout of S^T hands the weights to P^T
+        const int r16 = kk & 15;
+        const int slot = (kk & 16) + ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const __bf16 x = rv[r][e];
+          vt[(dv0 + e) * VP + slot] = *reinterpret_cast<const bf16s*>(&x);
+        }
+      }
+    }
+  };
 
   float m = -INFINITY, l = 0.0f;
   f32x16 oacc[VT];
@@ -200,72 +325,70 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[t][i] = 0.0f;
 
-  for (int it = 0; it < tiles; ++it) {
-    const bool sink = it < sink_tiles;
-    const int kbase = sink ? it * 32 : wstart + (it - sink_tiles) * 32;
-    const int klimit = sink ? n_sink : p1 + 1;  // keys of this tile at or above it are not this tile's to count
-    // S^T tile: rows = keys kbase..kbase+31, columns = the 32 tokens
-    const int jk = min(kbase + col, p1);
-    const long krow = ((long)bt[jk >> page_shift] << page_shift) + (jk & page_mask);
-    const bf16s* kr = kpool + (krow * G + g) * D + hf * 8;
-    f32x16 sacc;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int it = 0; it < tiles_n; ++it) {
+    const int buf = it & 1;
+    const bool more = it + 1 < tiles_n;
+    if (more) fetch(it + 1);
+    if (head_ok) {
+      const bool sink = it < sink_tiles;
+      const int kbase = tile_base(it);
+      const int klimit = sink ? n_sink : p1 + 1;  // keys of this tile at or above it are not this tile's to count
+      const bf16s* ks = tiles + buf * (KT + VTT);
+      const bf16s* vt = ks + KT;
+      f32x16 sacc;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
+      for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
 #pragma unroll
-    for (int s = 0; s < DS; ++s)
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld_g16b(kr + 16 * s), qf[s], sacc, 0, 0, 0);
-    float sv[16];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
-      const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
-      sv[i] = seen ? sacc[i] * scale - slope * (float)(pos - j) : -INFINITY;
-      tmax = fmaxf(tmax, sv[i]);
-    }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-    const float m_new = fmaxf(m, tmax);
-    const float corr = (m == -INFINITY) ? 1.0f : __expf(m - m_new);  // nothing accumulated yet: nothing to rescale
-    float psum = 0.0f;
-    bf16x8_v phi[2], plo[2];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float p = (sv[i] == -INFINITY) ? 0.0f : __expf(sv[i] - m_new);
-      psum += p;
-      const __bf16 hi = (__bf16)p;
-      phi[i >> 3][i & 7] = hi;
-      plo[i >> 3][i & 7] = (__bf16)(p - (float)hi);
-    }
-    l = l * corr + psum;
-    m = m_new;
-#pragma unroll
-    for (int t = 0; t < VT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[t][i] *= corr;
-    // O^T += V^T P^T: contraction slot (hf, e) of step s2 is key kbase + 16 s2 + 8 (e >> 2) + 4 hf + (e & 3)
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      long vrow[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int j = min(kbase + 16 * s2 + 8 * (e >> 2) + 4 * hf + (e & 3), p1);
-        vrow[e] = ((((long)bt[j >> page_shift] << page_shift) + (j & page_mask)) * G + g) * Dv + col;
+      for (int s = 0; s < DS; ++s) {
+        const bf16x8_v kf = *reinterpret_cast<const bf16x8_v*>(ks + col * KP + 16 * s + hf * 8);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc, 0, 0, 0);
       }
+      float sv[16];
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int t = 0; t < VT; ++t) {
-        bf16x8_v va;
+      for (int i = 0; i < 16; ++i) {
+        const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
+        const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
+        sv[i] = seen ? sacc[i] * scale - slope * (float)(pos - j) : -INFINITY;
+        tmax = fmaxf(tmax, sv[i]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+      const float m_new = fmaxf(m, tmax);
+      const float corr = (m == -INFINITY) ? 1.0f : __expf(m - m_new);  // nothing accumulated yet: nothing to rescale
+      float psum = 0.0f;
+      bf16x8_v phi[2], plo[2];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const bf16s raw = vpool[vrow[e] + t * 32];
-          va[e] = *reinterpret_cast<const __bf16*>(&raw);
+      for (int i = 0; i < 16; ++i) {
+        const float p = (sv[i] == -INFINITY) ? 0.0f : __expf(sv[i] - m_new);
+        psum += p;
+        const __bf16 hi = (__bf16)p;
+        phi[i >> 3][i & 7] = hi;
+        plo[i >> 3][i & 7] = (__bf16)(p - (float)hi);
+      }
+      l = l * corr + psum;
+      m = m_new;
+#pragma unroll
+      for (int t = 0; t < VT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[t][i] *= corr;
+      // O^T += V^T P^T: slot hf * 8 + e of step s2 holds key kbase + 16 s2 + 8 (e >> 2) + 4 hf + (e & 3)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+          const bf16x8_v va = *reinterpret_cast<const bf16x8_v*>(vt + (t * 32 + col) * VP + 16 * s2 + hf * 8);
+          oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, phi[s2], oacc[t], 0, 0, 0);
+          oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, plo[s2], oacc[t], 0, 0, 0);
         }
-        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, phi[s2], oacc[t], 0, 0, 0);
-        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, plo[s2], oacc[t], 0, 0, 0);
-      }
     }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
   }
   l += __shfl_xor(l, 32);
-  if (!tok_ok) return;
+  if (!tok_ok || !head_ok) return;
   float scale_out = 1.0f / l;
   if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h));
   bf16s* orow = out + (n * H + h) * (long)Dv;
@@ -293,7 +416,7 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   const int H = (int)q.size(1), D = (int)q.size(2);
   const int page = (int)kpool.size(1), G = (int)kpool.size(2), Dv = (int)vpool.size(3);
   TORCH_CHECK(kpool.size(3) == D && vpool.size(2) == G && vpool.size(1) == page && vpool.size(0) == kpool.size(0));
-  TORCH_CHECK(H % G == 0 && Dv <= 64 * MAX_VD_PER_LANE && page > 0 && (page & (page - 1)) == 0);
+  TORCH_CHECK(H % G == 0 && Dv <= 256 && page > 0 && (page & (page - 1)) == 0);
   check_i32(block_tables, "block_tables"); check_i32(tok_seq, "tok_seq"); check_i32(positions, "positions");
   TORCH_CHECK(block_tables.dim() == 2 && tok_seq.numel() == N && positions.numel() == N);
   TORCH_CHECK(window >= 0 && keep_first >= 0);
@@ -320,9 +443,11 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   const bool aligned = q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0;
   const bool mfma_shape = (D == 32 && Dv == 32) || ((D == 64 || D == 128) && (Dv == 64 || Dv == 128));
   if (num_tiles > 0 && is_bf16(q) && aligned && mfma_shape) {
-    const dim3 grid((unsigned)num_tiles, (unsigned)((H + 3) / 4));
+    const int rep = H / G, nw = 4;
+    const dim3 grid((unsigned)num_tiles, (unsigned)G, (unsigned)((rep + nw - 1) / nw));
+    const size_t msmem = (size_t)2 * (32 * (D + 8) + Dv * 40) * sizeof(bf16s);
 #define MFMA_CASE(DS_, VT_)                                                                                          \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<DS_, VT_>), grid, dim3(256), 0, stream(), ptr<bf16s>(out),        \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<DS_, VT_>), grid, dim3(64 * nw), msmem, stream(), ptr<bf16s>(out), \
                      ptr<bf16s>(q), (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool),                        \
                      block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu.data_ptr<int>(),                 \
                      start.data_ptr<int>(), slp, gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr,      \
@@ -336,15 +461,18 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
     HIP_CHECK_LAST();
     return out;
   }
-  const int Dp = (D + 3) & ~3;
-  const size_t smem = (size_t)(Dp + ATT_WAVES * 128 + ATT_WAVES * (2 + Dv)) * sizeof(float);
-  const int kvec = (is_bf16(q) ? D % 8 == 0 : D % 4 == 0) ? 1 : 0;
+  const int Dp = (D + 7) & ~7;
+  const int R = H / G, chunks = (R + RC - 1) / RC;
+  const size_t smem = (size_t)(RC * Dp + ATT_WAVES * (RC * 64 + 64) + ATT_WAVES * RC * (2 + Dv)) * sizeof(float);
+  TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
+  const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
+  const int vvec = Dv % 2 == 0 ? 1 : 0;
   SERVING_DISPATCH_ACT(q, T, {
-    hipLaunchKernelGGL(paged_attention_kernel<T>, dim3((unsigned)(N * H)), dim3(64 * ATT_WAVES), smem, stream(),
-                       ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),
+    hipLaunchKernelGGL(paged_attention_kernel<T>, dim3((unsigned)(N * G * chunks)), dim3(64 * ATT_WAVES), smem,
+                       stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),
                        block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),
                        positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride,
-                       H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec);
+                       H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec);
   });
   HIP_CHECK_LAST();
   return out;

@@ -100,7 +100,6 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
   constexpr int NOPS = DELTA ? 3 : 2;         // q, (k,) gate
   constexpr int CPB = 4 * 64 / P;             // value channels per block
   constexpr int OPF = CT * NOPS * Dp;         // operand floats per chunk
-  constexpr int R_OP = (OPF + 255) / 256;
   constexpr int R_V = (CT * CPB + 255) / 256;
   extern __shared__ __align__(16) float lds[];
   float* ops_buf = lds;                       // [2][CT][NOPS][Dp]
@@ -124,18 +123,33 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
 #pragma unroll
   for (int j = 0; j < DPL; ++j) S[j] = (!fresh && d0 + j < D) ? Sg[(long)(d0 + j) * Dv + cc] : 0.0f;
 
-  float r_op[R_OP], r_v[R_V], r_b = 0.0f;
+  // operand rows move as float4: a chunk is CT * NOPS rows of Dp / 4 float4 each
+  constexpr int RF4 = Dp / 4, OPF4 = CT * NOPS * RF4, R_OP4 = (OPF4 + 255) / 256;
+  float4v r_op[R_OP4];
+  float r_v[R_V], r_b = 0.0f;
+  const bool rows_vec = (D % 4) == 0;
+  const float* q_head = q + (long)hq * D;
+  const float* k_head = DELTA ? k + (long)hq * D : nullptr;
+  const float* g_head = gate + (long)h * D;
+  const long qk_stride = (long)Hq * D, g_stride = (long)H * D;
   auto fetch = [&](int tb) {  // chunk starting at token tb -> registers
 #pragma unroll
-    for (int r = 0; r < R_OP; ++r) {
+    for (int r = 0; r < R_OP4; ++r) {
       const int i = tid + 256 * r;
-      const int tok = i / (NOPS * Dp), op = (i / Dp) % NOPS, d = i % Dp;
-      const int t = tb + tok;
-      float val = (op == NOPS - 1) ? 1.0f : 0.0f;
-      if (i < OPF && t < t1 && d < D) {
-        if (op == NOPS - 1) val = gate[((long)t * H + h) * D + d];
-        else if (op == 0) val = q[((long)t * Hq + hq) * D + d];
-        else val = k[((long)t * Hq + hq) * D + d];
+      const int rowi = i / RF4, f4 = i % RF4;
+      const int tok = rowi / NOPS, op = rowi % NOPS;
+      const int t = tb + tok, d = f4 * 4;
+      const float fill = (op == NOPS - 1) ? 1.0f : 0.0f;
+      float4v val = {fill, fill, fill, fill};
+      if (i < OPF4 && t < t1 && d < D) {
+        const float* src = (op == NOPS - 1) ? g_head + t * g_stride : ((op == 0) ? q_head : k_head) + t * qk_stride;
+        if (rows_vec) {
+          val = *reinterpret_cast<const float4v*>(src + d);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (d + e < D) val[e] = src[d + e];
+        }
       }
       r_op[r] = val;
     }
@@ -148,11 +162,11 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
     }
     if (DELTA) r_b = (tid < CT && tb + tid < t1) ? beta[(long)(tb + tid) * H + h] : 0.0f;
   };
-  auto stash = [&](int buf) {  // registers -> LDS buffer
+  auto stash = [&](int buf) {  // registers -> LDS buffer ([CT][NOPS][Dp], the order the rows were fetched in)
 #pragma unroll
-    for (int r = 0; r < R_OP; ++r) {
+    for (int r = 0; r < R_OP4; ++r) {
       const int i = tid + 256 * r;
-      if (i < OPF) ops_buf[buf * OPF + i] = r_op[r];
+      if (i < OPF4) *reinterpret_cast<float4v*>(ops_buf + buf * OPF + i * 4) = r_op[r];
     }
 #pragma unroll
     for (int r = 0; r < R_V; ++r) {
@@ -185,30 +199,36 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
         gc[j] = gg[0]; gc[j + 1] = gg[1]; gc[j + 2] = gg[2]; gc[j + 3] = gg[3];
       }
       const float vc = v_buf[buf * CT * CPB + tt * CPB + cl];
-      float o = 0.0f;
+      const float bc = DELTA ? b_buf[buf * CT + tt] : 0.0f;
+      float oa = 0.0f, ob = 0.0f;  // two chains per sum: half the dependent depth
       if (DELTA) {
-        const float bc = b_buf[buf * CT + tt];
-        float dot = 0.0f;
+        float da = 0.0f, db = 0.0f;
 #pragma unroll
-        for (int j = 0; j < DPL; ++j) {
+        for (int j = 0; j < DPL; j += 2) {
           S[j] *= gc[j];
-          dot += S[j] * kc[j];
+          S[j + 1] *= gc[j + 1];
+          da += S[j] * kc[j];
+          db += S[j + 1] * kc[j + 1];
         }
-        dot = reduce_p<P>(dot);
+        const float dot = reduce_p<P>(da + db);
         const float u = bc * (vc - dot);
 #pragma unroll
-        for (int j = 0; j < DPL; ++j) {
+        for (int j = 0; j < DPL; j += 2) {
           S[j] += kc[j] * u;
-          o += S[j] * qc[j];
+          S[j + 1] += kc[j + 1] * u;
+          oa += S[j] * qc[j];
+          ob += S[j + 1] * qc[j + 1];
         }
       } else {
 #pragma unroll
-        for (int j = 0; j < DPL; ++j) {
+        for (int j = 0; j < DPL; j += 2) {
           S[j] = gc[j] * S[j] + (1.0f - gc[j]) * vc;
-          o += S[j] * qc[j];
+          S[j + 1] = gc[j + 1] * S[j + 1] + (1.0f - gc[j + 1]) * vc;
+          oa += S[j] * qc[j];
+          ob += S[j + 1] * qc[j + 1];
         }
       }
-      o = reduce_p<P>(o);
+      const float o = reduce_p<P>(oa + ob);
       if (p == 0 && live) out[((long)(tb + tt) * H + h) * Dv + c] = o;
     }
     if (more) stash(buf ^ 1);
