@@ -318,12 +318,17 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
   };
 
-  float m = -INFINITY, l = 0.0f;
+  float m = -INFINITY, l = 0.0f;  // m in the base-2 domain
   f32x16 oacc[VT];
 #pragma unroll
   for (int t = 0; t < VT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[t][i] = 0.0f;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float c1 = scale * LOG2E, sl2 = slope * LOG2E;
+  float row_bias[16];  // + slope log2e * (row of the C layout): the key's offset inside its tile
+#pragma unroll
+  for (int i = 0; i < 16; ++i) row_bias[i] = sl2 * (float)((i & 3) + 8 * (i >> 2) + 4 * hf);
 
   fetch(0);
   stash(0);
@@ -346,23 +351,36 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         const bf16x8_v kf = *reinterpret_cast<const bf16x8_v*>(ks + col * KP + 16 * s + hf * 8);
         sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc, 0, 0, 0);
       }
+      // scores in the base-2 domain: s2 = (q.k) scale log2e - slope log2e (pos - j), one add and one fma each
       float sv[16];
       float tmax = -INFINITY;
+      const float tile_bias = -sl2 * (float)(pos - kbase);
+      // interior tile: every key is visible to every token of the tile, no masks to evaluate
+      const bool interior = !sink && t_off + 31 < cnt && kbase + 31 <= p0 && (window == 0 || p1 - kbase < window);
+      if (interior) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
-        const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
-        sv[i] = seen ? sacc[i] * scale - slope * (float)(pos - j) : -INFINITY;
-        tmax = fmaxf(tmax, sv[i]);
+        for (int i = 0; i < 16; ++i) {
+          sv[i] = sacc[i] * c1 + (tile_bias + row_bias[i]);
+          tmax = fmaxf(tmax, sv[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
+          const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
+          sv[i] = seen ? sacc[i] * c1 + (tile_bias + row_bias[i]) : -INFINITY;
+          tmax = fmaxf(tmax, sv[i]);
+        }
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
       const float m_new = fmaxf(m, tmax);
-      const float corr = (m == -INFINITY) ? 1.0f : __expf(m - m_new);  // nothing accumulated yet: nothing to rescale
+      const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: every weight is exp2(-inf) = 0
+      const float corr = (m == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - m_new);  // nothing accumulated: nothing to rescale
       float psum = 0.0f;
       bf16x8_v phi[2], plo[2];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float p = (sv[i] == -INFINITY) ? 0.0f : __expf(sv[i] - m_new);
+        const float p = __builtin_amdgcn_exp2f(sv[i] - m_ref);
         psum += p;
         const __bf16 hi = (__bf16)p;
         phi[i >> 3][i & 7] = hi;
@@ -370,10 +388,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       }
       l = l * corr + psum;
       m = m_new;
+      if (!__all(corr == 1.0f)) {  // the running maxima of all 32 tokens stood still: no rescaling
 #pragma unroll
-      for (int t = 0; t < VT; ++t)
+        for (int t = 0; t < VT; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[t][i] *= corr;
+          for (int i = 0; i < 16; ++i) oacc[t][i] *= corr;
+      }
       // O^T += V^T P^T: slot hf * 8 + e of step s2 holds key kbase + 16 s2 + 8 (e >> 2) + 4 hf + (e & 3)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)

@@ -85,10 +85,13 @@ DEV_INLINE float reduce_p(float v) {
   return v;
 }
 
-// grid (ceil(Dv / (4 * 64 / P)), H, B), four waves per block; lane = (value channel, row slice p).
+// grid (ceil(Dv / (2 * 4 * 64 / P)), H, B), four waves per block; lane = (two value channels, row slice p).
 // q, k: [N, Hq, D] float (Hq = H / rep); gate: [N, H, D] float (decay g or forget f).
 // The block stages CT tokens' operand rows of its head in LDS (double-buffered: the next chunk's
 // global loads are in flight while this chunk's tokens are stepped through).
+// Every lane carries NC value channels (independent recurrences that share the operand reads):
+// their dependent chains interleave, which is what hides the LDS and DPP latencies when a long
+// prompt of one sequence leaves a single wave on a SIMD.
 template <int P, int DPL, bool DELTA, typename TV>
 __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ gate,
@@ -98,7 +101,9 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
   constexpr int Dp = P * DPL;                 // padded key size
   constexpr int CT = Dp > 128 ? 8 : 16;       // tokens per staged chunk
   constexpr int NOPS = DELTA ? 3 : 2;         // q, (k,) gate
-  constexpr int CPB = 4 * 64 / P;             // value channels per block
+  constexpr int NC = 2;                       // value channels per lane
+  constexpr int CPW = 4 * 64 / P;             // lanes groups (one channel each) per block
+  constexpr int CPB = CPW * NC;               // value channels per block
   constexpr int OPF = CT * NOPS * Dp;         // operand floats per chunk
   constexpr int R_V = (CT * CPB + 255) / 256;
   extern __shared__ __align__(16) float lds[];
@@ -110,18 +115,25 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int p = lane % P;
   const int cl = wid * (64 / P) + lane / P;   // channel inside the block
-  const int c = blockIdx.x * CPB + cl;
-  const bool live = c < Dv;
-  const int cc = live ? c : Dv - 1;
+  int c[NC], cc[NC];
+  bool live[NC];
+#pragma unroll
+  for (int x = 0; x < NC; ++x) {
+    c[x] = blockIdx.x * CPB + x * CPW + cl;
+    live[x] = c[x] < Dv;
+    cc[x] = live[x] ? c[x] : Dv - 1;
+  }
   const int d0 = p * DPL;
   const int Hq = H / rep, hq = h / rep;
   const int t0 = cu[b], t1 = cu[b + 1];
   float* Sg = state + (long)slots[b] * ss + (long)h * D * Dv;
 
-  float S[DPL];
+  float S[NC][DPL];
   const bool fresh = start[b] == 0;
 #pragma unroll
-  for (int j = 0; j < DPL; ++j) S[j] = (!fresh && d0 + j < D) ? Sg[(long)(d0 + j) * Dv + cc] : 0.0f;
+  for (int x = 0; x < NC; ++x)
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) S[x][j] = (!fresh && d0 + j < D) ? Sg[(long)(d0 + j) * Dv + cc[x]] : 0.0f;
 
   // operand rows move as float4: a chunk is CT * NOPS rows of Dp / 4 float4 each
   constexpr int RF4 = Dp / 4, OPF4 = CT * NOPS * RF4, R_OP4 = (OPF4 + 255) / 256;
@@ -198,47 +210,52 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
         const float4v gg = *reinterpret_cast<const float4v*>(row + (NOPS - 1) * Dp + j);
         gc[j] = gg[0]; gc[j + 1] = gg[1]; gc[j + 2] = gg[2]; gc[j + 3] = gg[3];
       }
-      const float vc = v_buf[buf * CT * CPB + tt * CPB + cl];
       const float bc = DELTA ? b_buf[buf * CT + tt] : 0.0f;
-      float oa = 0.0f, ob = 0.0f;  // two chains per sum: half the dependent depth
-      if (DELTA) {
-        float da = 0.0f, db = 0.0f;
 #pragma unroll
-        for (int j = 0; j < DPL; j += 2) {
-          S[j] *= gc[j];
-          S[j + 1] *= gc[j + 1];
-          da += S[j] * kc[j];
-          db += S[j + 1] * kc[j + 1];
-        }
-        const float dot = reduce_p<P>(da + db);
-        const float u = bc * (vc - dot);
+      for (int x = 0; x < NC; ++x) {
+        const float vc = v_buf[buf * CT * CPB + tt * CPB + x * CPW + cl];
+        float oa = 0.0f, ob = 0.0f;  // two chains per sum: half the dependent depth
+        if (DELTA) {
+          float da = 0.0f, db = 0.0f;
 #pragma unroll
-        for (int j = 0; j < DPL; j += 2) {
-          S[j] += kc[j] * u;
-          S[j + 1] += kc[j + 1] * u;
-          oa += S[j] * qc[j];
-          ob += S[j + 1] * qc[j + 1];
-        }
-      } else {
+          for (int j = 0; j < DPL; j += 2) {
+            S[x][j] *= gc[j];
+            S[x][j + 1] *= gc[j + 1];
+            da += S[x][j] * kc[j];
+            db += S[x][j + 1] * kc[j + 1];
+          }
+          const float dot = reduce_p<P>(da + db);
+          const float u = bc * (vc - dot);
 #pragma unroll
-        for (int j = 0; j < DPL; j += 2) {
-          S[j] = gc[j] * S[j] + (1.0f - gc[j]) * vc;
-          S[j + 1] = gc[j + 1] * S[j + 1] + (1.0f - gc[j + 1]) * vc;
-          oa += S[j] * qc[j];
-          ob += S[j + 1] * qc[j + 1];
+          for (int j = 0; j < DPL; j += 2) {
+            S[x][j] += kc[j] * u;
+            S[x][j + 1] += kc[j + 1] * u;
+            oa += S[x][j] * qc[j];
+            ob += S[x][j + 1] * qc[j + 1];
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < DPL; j += 2) {
+            S[x][j] = gc[j] * S[x][j] + (1.0f - gc[j]) * vc;
+            S[x][j + 1] = gc[j + 1] * S[x][j + 1] + (1.0f - gc[j + 1]) * vc;
+            oa += S[x][j] * qc[j];
+            ob += S[x][j + 1] * qc[j + 1];
+          }
         }
+        const float o = reduce_p<P>(oa + ob);
+        if (p == 0 && live[x]) out[((long)(tb + tt) * H + h) * Dv + c[x]] = o;
       }
-      const float o = reduce_p<P>(oa + ob);
-      if (p == 0 && live) out[((long)(tb + tt) * H + h) * Dv + c] = o;
     }
     if (more) stash(buf ^ 1);
     __syncthreads();
   }
-  if (live) {
 #pragma unroll
-    for (int j = 0; j < DPL; ++j)
-      if (d0 + j < D) Sg[(long)(d0 + j) * Dv + c] = S[j];
-  }
+  for (int x = 0; x < NC; ++x)
+    if (live[x]) {
+#pragma unroll
+      for (int j = 0; j < DPL; ++j)
+        if (d0 + j < D) Sg[(long)(d0 + j) * Dv + c[x]] = S[x][j];
+    }
 }
 
 template <bool DELTA, typename TV>
@@ -249,7 +266,7 @@ static void launch_scan(float* out, const float* q, const float* k, const float*
   const int dpl = D > 128 ? 16 : 8;
   int P = 1;
   while (P * dpl < D) P <<= 1;
-  const int cpb = 4 * 64 / P, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
+  const int cpb = 2 * 4 * 64 / P /* two channels per lane */, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
   const dim3 grid((unsigned)((Dv + cpb - 1) / cpb), (unsigned)H, (unsigned)B);
   const size_t smem = (size_t)(2 * ct * nops * Dp + 2 * ct * cpb + 2 * ct) * sizeof(float);
 #define SCAN_CASE(PP, DD)                                                                                          \
