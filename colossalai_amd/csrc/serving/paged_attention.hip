@@ -15,8 +15,8 @@
 namespace cai {
 namespace serving {
 
-constexpr int ATT_WAVES = 8;  // waves of a block: they split the key blocks of one (token, kv head)
-constexpr int RC = 4;         // query heads of the kv head's group handled together by a block
+constexpr int ATT_WAVES = 16;  // most waves of a block: they split the key blocks of one (token, kv head)
+constexpr int RC_MAX = 4;      // most query heads of a kv head's group that one block handles together
 
 template <int CTRL>
 DEV_INLINE float dpp_add(float v) {
@@ -48,25 +48,29 @@ DEV_INLINE void load2(const bf16s* p, float& a, float& b) {
 
 // Scalar kernel (decode tokens, float32 serving, shapes the MFMA kernel does not take).
 // One block per (token, kv head, group of up to RC query heads of that kv head): keys and
-// values are read once for the whole group. The block's waves take every ATT_WAVES-th block
-// of 64 keys and merge their partial softmax states through LDS at the end.
+// values are read once for the whole group. The block's nw waves (16, or 8 when the partial
+// states of 16 would not fit in LDS) take every nw-th block of 64 keys and merge their partial
+// softmax states through LDS at the end. The eight key steps of a block are unrolled so that
+// their page lookups and key loads are all in flight before the first product.
 // Scores: 8 adjacent lanes share a key, each takes a contiguous slice of the head size
 // (16-byte loads, few cache lines per instruction) and the slices are summed on the DPP path.
 // Values: lane = a pair of value channels, the block's weights and pool rows come from LDS.
-template <typename T>
+// RC = query heads per block: 4 shares each key/value read between the most heads; 2 or 1 are
+// chosen when a decode step would otherwise leave most CUs without a block (the re-reads hit L2).
+template <typename T, int RC>
 __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, const float* __restrict__ slopes, const T* __restrict__ gate, long gate_stride,
     int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec, int vvec) {
   extern __shared__ __align__(16) float lds[];
-  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const int Dp = (D + 7) & ~7;
   const int R = H / G, chunks = (R + RC - 1) / RC;
   float* qs = lds;                                        // [RC][Dp] queries
   float* pw = lds + RC * Dp + wid * (RC * 64 + 64);       // [RC][64] scores, then weights, of this wave's key block
   int* prow = reinterpret_cast<int*>(pw + RC * 64);       // [64] pool rows of the block
-  float* part = lds + RC * Dp + ATT_WAVES * (RC * 64 + 64);  // [waves][RC][2 + Dv] partial states
+  float* part = lds + RC * Dp + nw * (RC * 64 + 64);      // [waves][RC][2 + Dv] partial states
   const long n = blockIdx.x / (G * chunks);
   const int g = (int)(blockIdx.x / chunks) % G;
   const int h0 = g * R + (int)(blockIdx.x % chunks) * RC;  // first query head of this block
@@ -101,9 +105,9 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
   }
 
-  for (int base = wid * 64; base < total; base += 64 * ATT_WAVES) {
-#pragma unroll 2
-    for (int sub = 0; sub < 8; ++sub) {
+  for (int base = wid * 64; base < total; base += 64 * nw) {
+    const int cnt = min(64, total - base);
+    auto score_step = [&](int sub) {
       const int idx = base + sub * 8 + ksub;
       const bool valid = idx < total;
       const int j = valid ? (idx < n_keep ? idx : lo + (idx - n_keep)) : pos;
@@ -139,13 +143,19 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
           pw[r * 64 + sub * 8 + ksub] = valid ? dots[r] * scale - slope[r] * (float)(pos - j) : -INFINITY;
         prow[sub * 8 + ksub] = row;
       }
+    };
+    if (cnt == 64) {  // straight-line: all eight steps' lookups and key loads issue before the first product
+#pragma unroll
+      for (int sub = 0; sub < 8; ++sub) score_step(sub);
+    } else {          // the last block of a key range: only the steps that hold keys
+      for (int sub = 0; sub * 8 < cnt; ++sub) score_step(sub);
     }
     // the wave is its own producer and consumer of pw/prow: wait for its LDS writes
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     float corr[RC];
 #pragma unroll
     for (int r = 0; r < RC; ++r) {
-      const float s = pw[r * 64 + lane];
+      const float s = lane < cnt ? pw[r * 64 + lane] : -INFINITY;
       const float m_new = fmaxf(m[r], wave_reduce_max(s));  // a block holds at least one visible key
       const float w = expf(s - m_new);                      // exp(-inf) = 0 for the block's empty places
       corr[r] = expf(m[r] - m_new);                         // m = -inf before the first block: 0
@@ -158,9 +168,8 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     for (int r = 0; r < RC; ++r)
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[r][i] *= corr[r];
-    const int cnt = min(64, total - base);
     const int dva = 2 * lane, dvb = 128 + 2 * lane;
-#pragma unroll 4
+#pragma unroll 8
     for (int jj = 0; jj < cnt; ++jj) {
       const T* vr = vpool + ((long)prow[jj] * G + g) * Dv;
       float v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
@@ -196,9 +205,9 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
   for (int i = threadIdx.x; i < nh * Dv; i += blockDim.x) {
     const int r = i / Dv, dv = i % Dv;
     float mm = -INFINITY;
-    for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, part[(w * RC + r) * PS]);
+    for (int w = 0; w < nw; ++w) mm = fmaxf(mm, part[(w * RC + r) * PS]);
     float ll = 0.0f, o = 0.0f;
-    for (int w = 0; w < ATT_WAVES; ++w) {
+    for (int w = 0; w < nw; ++w) {
       const float mw = part[(w * RC + r) * PS];
       if (mw != -INFINITY) {
         const float f = expf(mw - mm);
@@ -482,18 +491,28 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
     return out;
   }
   const int Dp = (D + 7) & ~7;
-  const int R = H / G, chunks = (R + RC - 1) / RC;
-  const size_t smem = (size_t)(RC * Dp + ATT_WAVES * (RC * 64 + 64) + ATT_WAVES * RC * (2 + Dv)) * sizeof(float);
+  const int R = H / G;
+  int rc = RC_MAX;
+  while (rc > 1 && (rc > R || N * G * ((R + rc - 1) / rc) < 256)) rc >>= 1;  // enough blocks to cover the CUs
+  const int chunks = (R + rc - 1) / rc;
+  auto lds_bytes = [&](int nw) { return (size_t)(rc * Dp + nw * (rc * 64 + 64) + nw * rc * (2 + Dv)) * sizeof(float); };
+  const int nwaves = lds_bytes(ATT_WAVES) <= 64 * 1024 ? ATT_WAVES : ATT_WAVES / 2;
+  const size_t smem = lds_bytes(nwaves);
   TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
   const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
   const int vvec = Dv % 2 == 0 ? 1 : 0;
+#define SCALAR_CASE(RC_)                                                                                            \
+  hipLaunchKernelGGL((paged_attention_kernel<T, RC_>), dim3((unsigned)(N * G * chunks)), dim3(64 * nwaves), smem,   \
+                     stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),             \
+                     block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),            \
+                     positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride, \
+                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec)
   SERVING_DISPATCH_ACT(q, T, {
-    hipLaunchKernelGGL(paged_attention_kernel<T>, dim3((unsigned)(N * G * chunks)), dim3(64 * ATT_WAVES), smem,
-                       stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),
-                       block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),
-                       positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride,
-                       H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec);
+    if (rc == 4) SCALAR_CASE(4);
+    else if (rc == 2) SCALAR_CASE(2);
+    else SCALAR_CASE(1);
   });
+#undef SCALAR_CASE
   HIP_CHECK_LAST();
   return out;
 }

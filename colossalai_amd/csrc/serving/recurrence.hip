@@ -85,13 +85,14 @@ DEV_INLINE float reduce_p(float v) {
   return v;
 }
 
-// grid (ceil(Dv / (2 * 4 * 64 / P)), H, B), four waves per block; lane = (two value channels, row slice p).
+// grid (ceil(Dv / (4 * 64 / P)), H, B), four waves per block; lane = (value channel, row slice p).
 // q, k: [N, Hq, D] float (Hq = H / rep); gate: [N, H, D] float (decay g or forget f).
 // The block stages CT tokens' operand rows of its head in LDS (double-buffered: the next chunk's
 // global loads are in flight while this chunk's tokens are stepped through).
-// Every lane carries NC value channels (independent recurrences that share the operand reads):
-// their dependent chains interleave, which is what hides the LDS and DPP latencies when a long
-// prompt of one sequence leaves a single wave on a SIMD.
+// A lane can carry NC value channels that share the operand reads. Measured on a 4096-token
+// prompt (D = 128): NC = 2 is 1.5x slower per layer than NC = 1 - a single long sequence is
+// bound by the instructions a wave issues per token, not by latencies that a second chain could
+// hide - so NC stays 1.
 template <int P, int DPL, bool DELTA, typename TV>
 __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ gate,
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
   constexpr int Dp = P * DPL;                 // padded key size
   constexpr int CT = Dp > 128 ? 8 : 16;       // tokens per staged chunk
   constexpr int NOPS = DELTA ? 3 : 2;         // q, (k,) gate
-  constexpr int NC = 2;                       // value channels per lane
+  constexpr int NC = 1;                       // value channels per lane
   constexpr int CPW = 4 * 64 / P;             // lanes groups (one channel each) per block
   constexpr int CPB = CPW * NC;               // value channels per block
   constexpr int OPF = CT * NOPS * Dp;         // operand floats per chunk
@@ -266,7 +267,7 @@ static void launch_scan(float* out, const float* q, const float* k, const float*
   const int dpl = D > 128 ? 16 : 8;
   int P = 1;
   while (P * dpl < D) P <<= 1;
-  const int cpb = 2 * 4 * 64 / P /* two channels per lane */, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
+  const int cpb = 4 * 64 / P /* times NC of the kernel */, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
   const dim3 grid((unsigned)((Dv + cpb - 1) / cpb), (unsigned)H, (unsigned)B);
   const size_t smem = (size_t)(2 * ct * nops * Dp + 2 * ct * cpb + 2 * ct) * sizeof(float);
 #define SCAN_CASE(PP, DD)                                                                                          \

@@ -145,7 +145,7 @@ def test_tied_gate_recurrence(dtype, H, D, Dv):
 @pytest.mark.parametrize("page", [16, 64])
 @pytest.mark.parametrize("H,G,D,Dv,window,keep", [(4, 2, 32, 32, 9, 3), (6, 3, 24, 40, 0, 0), (2, 2, 64, 16, 70, 0),
                                                   (4, 1, 16, 130, 5, 30), (8, 2, 64, 64, 40, 20), (5, 5, 128, 128, 0, 0),
-                                                  (4, 2, 128, 64, 33, 2), (2, 1, 64, 128, 31, 40)])
+                                                  (4, 2, 128, 64, 33, 2), (2, 1, 64, 128, 31, 40), (8, 1, 64, 64, 12, 1)])
 def test_paged_attention(dtype, H, G, D, Dv, window, keep, page):
     """Scalar kernel (float32, odd head sizes) and matrix-core kernel (bfloat16
     with head sizes it tiles) on the same ragged batch; the pool's other rows
@@ -182,3 +182,26 @@ def test_activations():
     xb = x.bfloat16()
     torch.testing.assert_close(relu_squared(xb.cuda()).cpu(), torch.relu(xb).square())
     torch.testing.assert_close(softcap(x.cuda() * 20, 15.0).cpu(), 15.0 * torch.tanh(x * 20 / 15.0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("counts", [[200, 100], [90, 60], [7, 3]])
+def test_paged_attention_heads_per_block(counts):
+    """The scalar kernel picks how many query heads of a group share a block
+    from the size of the step (4, 2 or 1): all three must agree with the
+    reference (float32, 4 query heads on one kv head)."""
+    torch.manual_seed(8)
+    H, G, D, Dv, page = 4, 1, 24, 20, 16
+    starts = [5, 0]
+    tables, nxt = [], 0
+    for c, s in zip(counts, starts):
+        need = (c + s + page - 1) // page
+        tables.append(list(range(nxt, nxt + need)))
+        nxt += need
+    gb = RaggedBatch.build(counts, starts, [0, 1], "cuda", tables, page)
+    cb = RaggedBatch.build(counts, starts, [0, 1], "cpu", tables, page)
+    kpool, vpool = torch.randn(nxt, page, G, D), torch.randn(nxt, page, G, Dv)
+    q = torch.randn(gb.num_tokens, H, D)
+    slopes = paged_attention.distance_slopes(H)
+    out = paged_attention.paged_attention(q.cuda(), kpool.cuda(), vpool.cuda(), gb, 0.3, 50, 3, slopes.cuda(), None)
+    ref = paged_attention.paged_attention_ref(q, kpool, vpool, cb, 0.3, 50, 3, slopes, None)
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-4)
