@@ -16,7 +16,7 @@ at::Tensor head_rms_norm_gate(at::Tensor x, at::Tensor weight, double eps, c10::
 at::Tensor merge_rms_norm(at::Tensor a, at::Tensor wa, at::Tensor b, at::Tensor wb, double eps, at::Tensor out_w,
                           int64_t groups, at::Tensor residual);
 at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> tail, at::Tensor cu, at::Tensor start,
-                      at::Tensor slots, at::Tensor tok_seq, bool silu);
+                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype);
 at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta_logit, at::Tensor dt,
                             at::Tensor A_log, at::Tensor dt_bias, at::Tensor state, at::Tensor cu, at::Tensor start,
                             at::Tensor slots, double unit_eps, double q_scale);

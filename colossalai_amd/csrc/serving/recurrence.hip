@@ -23,11 +23,12 @@ namespace serving {
 
 // ------------------------------------------------------------------ prologue
 // One block per token. q/k [N, G, D] row-strided; dt [N, H*D] row-strided.
-template <typename T>
+// T: type of q/k (the convolution's output), TL: type of the gate and decay logits (projections).
+template <typename T, typename TL>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
     float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ dec, float* __restrict__ beta,
-    const T* __restrict__ q, long qs, const T* __restrict__ k, long ks, const T* __restrict__ bl, long bs,
-    const T* __restrict__ dt, long ds, const float* __restrict__ A_log, const float* __restrict__ dt_bias, int G, int H,
+    const T* __restrict__ q, long qs, const T* __restrict__ k, long ks, const TL* __restrict__ bl, long bs,
+    const TL* __restrict__ dt, long ds, const float* __restrict__ A_log, const float* __restrict__ dt_bias, int G, int H,
     int D, float unit_eps, float q_scale) {
   const long n = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -305,7 +306,7 @@ at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor
   TORCH_CHECK(beta_logit.dim() == 2 && beta_logit.size(0) == N && beta_logit.size(1) == H && beta_logit.stride(1) == 1);
   TORCH_CHECK(dt.dim() == 2 && dt.size(0) == N && dt.size(1) == (long)H * D && dt.stride(1) == 1);
   TORCH_CHECK(q.scalar_type() == k.scalar_type() && q.scalar_type() == v.scalar_type() &&
-              q.scalar_type() == beta_logit.scalar_type() && q.scalar_type() == dt.scalar_type());
+              beta_logit.scalar_type() == dt.scalar_type(), "q/k/v share one dtype, the logits another or the same");
   check_state(state, H, D, Dv);
   check_i32(cu, "cu"); check_i32(start, "start"); check_i32(slots, "slots");
   const int B = (int)start.numel();
@@ -317,11 +318,13 @@ at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor
   at::Tensor qn = at::empty({N, G, D}, fo), kn = at::empty({N, G, D}, fo), dec = at::empty({N, H, D}, fo),
              beta = at::empty({N, H}, fo);
   SERVING_DISPATCH_ACT(q, T, {
-    hipLaunchKernelGGL(delta_prepare_kernel<T>, dim3((unsigned)N), dim3(256), 0, stream(), qn.data_ptr<float>(),
-                       kn.data_ptr<float>(), dec.data_ptr<float>(), beta.data_ptr<float>(), ptr<T>(q),
-                       (long)q.stride(0), ptr<T>(k), (long)k.stride(0), ptr<T>(beta_logit), (long)beta_logit.stride(0),
-                       ptr<T>(dt), (long)dt.stride(0), Af.data_ptr<float>(), bf.data_ptr<float>(), G, H, D,
-                       (float)unit_eps, (float)q_scale);
+    SERVING_DISPATCH_ACT(dt, TL, {
+      hipLaunchKernelGGL((delta_prepare_kernel<T, TL>), dim3((unsigned)N), dim3(256), 0, stream(), qn.data_ptr<float>(),
+                         kn.data_ptr<float>(), dec.data_ptr<float>(), beta.data_ptr<float>(), ptr<T>(q),
+                         (long)q.stride(0), ptr<T>(k), (long)k.stride(0), ptr<TL>(beta_logit),
+                         (long)beta_logit.stride(0), ptr<TL>(dt), (long)dt.stride(0), Af.data_ptr<float>(),
+                         bf.data_ptr<float>(), G, H, D, (float)unit_eps, (float)q_scale);
+    });
     HIP_CHECK_LAST();
     launch_scan<true, T>(out.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(), dec.data_ptr<float>(),
                          beta.data_ptr<float>(), ptr<T>(v), (long)v.stride(0), state.data_ptr<float>(),

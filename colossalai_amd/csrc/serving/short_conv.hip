@@ -14,9 +14,9 @@ constexpr int MAX_TAPS = 16;
 
 // x element (n, c) at n*xs + c. tail element (slot, r, c) at slot*ts + r*C + c,
 // r = 0 oldest .. K-2 the token just before the portion.
-template <typename T>
+template <typename T, typename TO>
 __global__ __launch_bounds__(256) void short_conv_kernel(
-    T* __restrict__ y, const T* __restrict__ x, long xs, const float* __restrict__ taps, const float* __restrict__ tail,
+    TO* __restrict__ y, const T* __restrict__ x, long xs, const float* __restrict__ taps, const float* __restrict__ tail,
     long ts, const int* __restrict__ cu, const int* __restrict__ start, const int* __restrict__ slots,
     const int* __restrict__ tok_seq, int C, int K, int silu) {
   const int n = blockIdx.x;
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void short_conv_tail_kernel(
 }
 
 at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> tail, at::Tensor cu, at::Tensor start,
-                      at::Tensor slots, at::Tensor tok_seq, bool silu) {
+                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype) {
   check_act(x, "x");
   TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1, "x must be [N, C] with unit inner stride");
   const long N = x.size(0);
@@ -72,7 +72,7 @@ at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> t
   check_i32(cu, "cu"); check_i32(start, "start"); check_i32(slots, "slots"); check_i32(tok_seq, "tok_seq");
   TORCH_CHECK(tok_seq.numel() == N);
   at::Tensor tp = f32c(taps);
-  at::Tensor y = at::empty({N, C}, x.options());
+  at::Tensor y = at::empty({N, C}, x.options().dtype(out_dtype));
   if (N == 0) return y;
   const float* tlp = nullptr;
   float* tlw = nullptr;
@@ -88,9 +88,11 @@ at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> t
   const int B = (int)start.numel();
   const unsigned gy = (unsigned)((C + 255) / 256);
   SERVING_DISPATCH_ACT(x, T, {
-    hipLaunchKernelGGL(short_conv_kernel<T>, dim3((unsigned)N, gy), dim3(256), 0, stream(), ptr<T>(y), ptr<T>(x),
-                       (long)x.stride(0), tp.data_ptr<float>(), tlp, ts, cu.data_ptr<int>(), start.data_ptr<int>(),
-                       slots.data_ptr<int>(), tok_seq.data_ptr<int>(), C, K, (int)silu);
+    SERVING_DISPATCH_ACT(y, TO, {
+      hipLaunchKernelGGL((short_conv_kernel<T, TO>), dim3((unsigned)N, gy), dim3(256), 0, stream(), ptr<TO>(y), ptr<T>(x),
+                         (long)x.stride(0), tp.data_ptr<float>(), tlp, ts, cu.data_ptr<int>(), start.data_ptr<int>(),
+                         slots.data_ptr<int>(), tok_seq.data_ptr<int>(), C, K, (int)silu);
+    });
     if (K > 1)
       hipLaunchKernelGGL(short_conv_tail_kernel<T>, dim3((unsigned)B, gy), dim3(256), 0, stream(), ptr<T>(x),
                          (long)x.stride(0), tlw, ts, cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(),

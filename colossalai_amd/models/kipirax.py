@@ -176,7 +176,8 @@ class KipiraxChannelDeltaMixer(nn.Module):
     def forward(self, h, batch: RaggedBatch, kpool, vpool, state, norm_w, groups, residual):
         N = h.shape[0]
         p, y = self.in_proj(h)
-        qkv = short_conv(y[:, : self.C], self.conv, state.get("tail"), batch, True)
+        # the convolution feeds a recurrence: its activated output stays float32
+        qkv = short_conv(y[:, : self.C], self.conv, state.get("tail"), batch, True, torch.float32)
         q = qkv[:, : self.Cq].view(N, self.G, self.D)
         k = qkv[:, self.Cq : 2 * self.Cq].view(N, self.G, self.D)
         v = qkv[:, 2 * self.Cq :].view(N, self.H, self.Dv)

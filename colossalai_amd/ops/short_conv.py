@@ -15,9 +15,9 @@ from .ragged import RaggedBatch
 __all__ = ["short_conv", "short_conv_ref"]
 
 
-def short_conv_ref(x, taps, tail, batch: RaggedBatch, silu: bool = True):
+def short_conv_ref(x, taps, tail, batch: RaggedBatch, silu: bool = True, out_dtype=None):
     K = taps.shape[1]
-    y = torch.empty_like(x)
+    y = torch.empty_like(x, dtype=out_dtype or x.dtype)
     tf = taps.float()
     for i in range(batch.num_seqs):
         lo, hi, slot = batch.cu_host[i], batch.cu_host[i + 1], batch.slots_host[i]
@@ -31,14 +31,17 @@ def short_conv_ref(x, taps, tail, batch: RaggedBatch, silu: bool = True):
         acc = torch.zeros(hi - lo, x.shape[1], device=x.device)
         for j in range(K):
             acc = acc + full[j : j + hi - lo] * tf[:, j]
-        y[lo:hi] = (F.silu(acc) if silu else acc).to(x.dtype)
+        y[lo:hi] = (F.silu(acc) if silu else acc).to(y.dtype)
         if K > 1:
             tail[slot] = full[full.shape[0] - (K - 1):]
     return y
 
 
-def short_conv(x, taps, tail, batch: RaggedBatch, silu: bool = True):
-    """x [N, C], taps [C, K], tail [slots, K-1, C] float32 (slot-strided allowed)."""
+def short_conv(x, taps, tail, batch: RaggedBatch, silu: bool = True, out_dtype=None):
+    """x [N, C], taps [C, K], tail [slots, K-1, C] float32 (slot-strided allowed).
+    The sum and the activation are float32; ``out_dtype`` (default: x's) is what
+    the result is stored in — float32 keeps a recurrence's inputs unrounded."""
     if use_hip(x):
-        return serving_kernels().short_conv(x, taps, tail, batch.cu, batch.start, batch.slots, batch.tok_seq, silu)
-    return short_conv_ref(x, taps, tail, batch, silu)
+        return serving_kernels().short_conv(x, taps, tail, batch.cu, batch.start, batch.slots, batch.tok_seq, silu,
+                                            out_dtype or x.dtype)
+    return short_conv_ref(x, taps, tail, batch, silu, out_dtype)

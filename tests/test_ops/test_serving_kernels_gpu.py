@@ -100,18 +100,27 @@ def test_short_conv(dtype, K):
     tc = arena.clone()[:, : (K - 1) * C].view(6, K - 1, C) if K > 1 else None
     out = short_conv.short_conv(wide.cuda()[:, :C], taps.cuda(), tg, gb, True)
     ref = short_conv.short_conv_ref(wide[:, :C], taps, tc, cb, True)
+    assert out.dtype == dtype
     torch.testing.assert_close(out.cpu().float(), ref.float(), **tol(dtype))
+    if K > 1:  # float32 output of the same inputs (the slot's tail is refreshed again: same values)
+        wide32 = short_conv.short_conv(wide.cuda()[:, :C], taps.cuda(), tg.clone(), gb, True, torch.float32)
+        assert wide32.dtype == torch.float32
+        torch.testing.assert_close(wide32.cpu(), short_conv.short_conv_ref(wide[:, :C], taps, tc.clone(), cb, True, torch.float32),
+                                   rtol=2e-5, atol=2e-5)
     if K > 1:
         torch.testing.assert_close(tg.cpu(), tc, **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 24), (3, 3, 20, 64), (2, 1, 128, 70), (2, 2, 8, 8)])
-def test_gated_delta_rule(dtype, H, G, D, Dv):
+@pytest.mark.parametrize("qkv32", [False, True])
+def test_gated_delta_rule(dtype, H, G, D, Dv, qkv32):
+    """qkv32: q/k/v arrive in float32 (an unrounded convolution output) next to logits in ``dtype``."""
     torch.manual_seed(4)
     gb, cb, _ = make_batch("cuda")
     N = gb.num_tokens
-    q, k, v = (torch.randn(N, G, D).to(dtype), torch.randn(N, G, D).to(dtype), torch.randn(N, H, Dv).to(dtype))
+    qd = torch.float32 if qkv32 else dtype
+    q, k, v = (torch.randn(N, G, D).to(qd), torch.randn(N, G, D).to(qd), torch.randn(N, H, Dv).to(qd))
     bl, dt = torch.randn(N, H).to(dtype), torch.randn(N, H * D).to(dtype)
     A, bias = torch.randn(H) - 1, torch.randn(H * D)
     state = torch.randn(6, H, D, Dv)
