@@ -28,11 +28,16 @@ class KVCacheManager:
         device=None,
         dtype=torch.bfloat16,
         layer_shapes: Optional[List[Optional[tuple]]] = None,
+        layer_sources: Optional[List[Optional[int]]] = None,
     ):
         """``layer_shapes`` (optional) gives each layer its own
         ``(kv_heads, key_dim, value_dim)`` or ``None`` for a layer that keeps no
         keys (a recurrent layer of a hybrid model); without it every layer gets
-        ``(num_kv_heads, head_dim, head_dim)``."""
+        ``(num_kv_heads, head_dim, head_dim)``. ``layer_sources`` (optional)
+        names, for a layer that projects no keys of its own, the layer whose
+        pools it reads: ``k_pools[i]`` / ``v_pools[i]`` are then that layer's
+        tensors (no second copy; the pages and page tables are shared by all
+        layers anyway), and the layer's own shape entry must be ``None``."""
         assert block_size & (block_size - 1) == 0, "block_size must be a power of two"
         self.num_layers = num_layers
         self.block_size = block_size
@@ -50,6 +55,14 @@ class KVCacheManager:
             None if s is None else torch.zeros(num_blocks, block_size, s[0], s[2], device=self.device, dtype=dtype)
             for s in layer_shapes
         ]
+        self.layer_sources = list(layer_sources) if layer_sources is not None else [None] * num_layers
+        assert len(self.layer_sources) == num_layers
+        for i, src in enumerate(self.layer_sources):
+            if src is not None:
+                assert layer_shapes[i] is None, f"layer {i} reads layer {src}'s pools and keeps none of its own"
+                assert self.layer_sources[src] is None and self.k_pools[src] is not None, \
+                    f"layer {i} reads keys of layer {src}, which keeps none"
+                self.k_pools[i], self.v_pools[i] = self.k_pools[src], self.v_pools[src]
         self._free: List[int] = list(range(num_blocks - 1, -1, -1))
         self._tables: Dict[int, List[int]] = {}  # seq id -> block ids
 

@@ -43,6 +43,7 @@ from ..ops.ragged import RaggedBatch
 from ..ops.short_conv import short_conv
 from ..ops.token_shift import token_shift
 from ..ops.activation import relu_squared, softcap
+from .packed import PackedLinear as _Packed
 from .registry import register_model
 
 __all__ = ["KipiraxConfig", "KipiraxForCausalLM"]
@@ -74,25 +75,6 @@ class KipiraxConfig:
 
 def _vec(n, value=1.0):
     return nn.Parameter(torch.full((n,), value, dtype=torch.float32))
-
-
-class _Packed(nn.Module):
-    """Several ``[out_i, in]`` projections stored as one matrix; ``split`` hands
-    back column views of the single GEMM's output."""
-
-    def __init__(self, in_features: int, parts: Dict[str, int]):
-        super().__init__()
-        self.parts = dict(parts)
-        self.offsets, at = {}, 0
-        for name, n in parts.items():
-            self.offsets[name] = (at, at + n)
-            at += n
-        self.weight = nn.Parameter(torch.empty(at, in_features))
-        nn.init.normal_(self.weight, std=in_features ** -0.5)
-
-    def forward(self, h):
-        y = F.linear(h, self.weight)
-        return {name: y[:, lo:hi] for name, (lo, hi) in self.offsets.items()}, y
 
 
 class KipiraxParallelMixer(nn.Module):

@@ -1,20 +1,31 @@
 """Small element-wise activations of the serving path.
 
-``relu_squared(x) = max(x, 0)^2`` (feed-forward activation) and
-``softcap(x, c) = c * tanh(x / c)`` (bounded logits, float32).
+``relu_squared(x) = max(x, 0)^2`` (feed-forward activation),
+``silu_mul([g | u]) = g * sigmoid(g) * u`` on a packed ``[N, 2F]`` tensor (gated
+feed-forward) and ``softcap(x, c) = c * tanh(x / c)`` (bounded logits, float32).
 """
 
 import torch
 
 from ._kernels import serving_kernels, use_serving_hip
 
-__all__ = ["relu_squared", "softcap"]
+__all__ = ["relu_squared", "silu_mul", "softcap"]
 
 
 def relu_squared(x: torch.Tensor) -> torch.Tensor:
     if use_serving_hip(x) and not torch.is_grad_enabled():
         return serving_kernels().relu_squared(x.contiguous())
     return torch.relu(x).square()
+
+
+def silu_mul(packed: torch.Tensor) -> torch.Tensor:
+    """packed [N, 2F] = [gate | up] (rows may be strided) -> [N, F]; the product
+    is formed in float32 and rounded once."""
+    F_ = packed.shape[-1] // 2
+    if use_serving_hip(packed) and not torch.is_grad_enabled():
+        return serving_kernels().silu_mul(packed)
+    g, u = packed[..., :F_].float(), packed[..., F_:].float()
+    return (g * torch.sigmoid(g) * u).to(packed.dtype)
 
 
 def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:

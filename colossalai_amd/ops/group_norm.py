@@ -6,7 +6,9 @@ element-wise weight; with ``residual`` it adds the result to a float32 residual
 stream in place (norm on the sublayer's *output*). ``groups=1`` is plain RMS
 norm. ``head_rms_norm_gate`` normalises every head vector of a ``[N, H, D]``
 tensor with one shared ``[D]`` weight and optionally multiplies by
-``sigmoid(gate)``. All statistics are float32.
+``sigmoid(gate)``. ``add_rms_norm`` serves pre-norm layers: it adds one or two
+sublayer outputs to the float32 residual stream in place and hands back the
+RMS-normed stream for the next layer in one pass. All statistics are float32.
 """
 
 from typing import Optional
@@ -16,7 +18,7 @@ import torch
 from ._kernels import serving_kernels, use_serving_hip as use_hip
 
 __all__ = ["grouped_rms_norm", "grouped_rms_norm_ref", "head_rms_norm_gate", "head_rms_norm_gate_ref",
-           "merge_rms_norm", "merge_rms_norm_ref"]
+           "merge_rms_norm", "merge_rms_norm_ref", "add_rms_norm", "add_rms_norm_ref"]
 
 
 def grouped_rms_norm_ref(x, weight, groups: int, eps: float, residual=None, out_dtype=None):
@@ -69,3 +71,22 @@ def merge_rms_norm(a, wa, b, wb, eps: float, out_w, groups: int, residual):
     if use_hip(a):
         return serving_kernels().merge_rms_norm(a.contiguous(), wa, b.contiguous(), wb, eps, out_w, groups, residual)
     return merge_rms_norm_ref(a, wa, b, wb, eps, out_w, groups, residual)
+
+
+def add_rms_norm_ref(residual, a, b, weight, eps: float, out_dtype=None):
+    residual.add_(a.float() if b is None else a.float() + b.float())
+    if weight is None:
+        return None
+    return grouped_rms_norm_ref(residual, weight, 1, eps, None, out_dtype or a.dtype)
+
+
+def add_rms_norm(residual, a, b, weight, eps: float, out_dtype=None):
+    """``residual += a (+ b)`` in place (float32 [N, W]; ``a``/``b`` sublayer
+    outputs of any activation type, ``b`` may be None), then, when ``weight`` is
+    given, returns ``rms_norm(residual) * weight`` in ``out_dtype`` — the input
+    of the next pre-norm layer. With ``weight=None`` only the sum is formed."""
+    if use_hip(residual):
+        assert residual.dtype == torch.float32
+        return serving_kernels().add_rms_norm(residual, a.contiguous(), None if b is None else b.contiguous(),
+                                              weight, eps, out_dtype or a.dtype)
+    return add_rms_norm_ref(residual, a, b, weight, eps, out_dtype)

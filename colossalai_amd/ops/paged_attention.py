@@ -9,7 +9,12 @@ keys (``paged_kv_write`` runs first). Masking and bias are parameters:
   visible (attention sinks that keep their true positions);
 * an optional per-head linear distance penalty ``slopes[h] * (i - j)`` taken
   off the scaled score;
-* an optional per-head output gate ``sigmoid(gate[n, h])``.
+* an optional per-head output gate ``sigmoid(gate[n, h])``;
+* an optional soft cap ``softcap * tanh(score / softcap)`` on the scaled score
+  (before the distance penalty);
+* an optional *sink*: one more place of score 0 in the softmax denominator that
+  carries no value, ``p_j = exp(s_j) / (1 + sum exp(s_j))``, so a query may
+  attend to nothing.
 
 Scores, softmax weights and the accumulation are float32. Key and value head
 sizes may differ; query head ``h`` reads key/value head ``h // (H / G)``.
@@ -43,7 +48,8 @@ def paged_kv_write(k, v, kpool, vpool, batch: RaggedBatch):
 
 
 def paged_attention_ref(q, kpool, vpool, batch: RaggedBatch, scale: float, window: int = 0, keep_first: int = 0,
-                        slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None):
+                        slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                        softcap: float = 0.0, sink: bool = False):
     N, H, D = q.shape
     G, Dv = vpool.shape[2], vpool.shape[3]
     ps = kpool.shape[1]
@@ -58,24 +64,30 @@ def paged_attention_ref(q, kpool, vpool, batch: RaggedBatch, scale: float, windo
         kj = torch.arange(L, device=q.device)[None, :]
         dist = (qi - kj).float()
         s = torch.einsum("nhd,lhd->hnl", q[lo:hi].float(), kk) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
         if slopes is not None:
             s = s - slopes.float()[:, None, None] * dist
         seen = kj <= qi
         if window > 0:
             seen = seen & ((qi - kj < window) | (kj < keep_first))
         s = s.masked_fill(~seen, float("-inf"))
-        out[lo:hi] = torch.einsum("hnl,lhv->nhv", torch.softmax(s, -1), vv)
+        if sink:  # a zero-score column without a value
+            s = torch.cat([s, torch.zeros_like(s[..., :1])], -1)
+        p = torch.softmax(s, -1)[..., :L]
+        out[lo:hi] = torch.einsum("hnl,lhv->nhv", p, vv)
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[:, :, None]
     return out.to(q.dtype)
 
 
 def paged_attention(q, kpool, vpool, batch: RaggedBatch, scale: float, window: int = 0, keep_first: int = 0,
-                    slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None):
+                    slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                    softcap: float = 0.0, sink: bool = False):
     """q [N, H, D]; returns [N, H, Dv] in q's dtype. ``window == 0`` means no
-    window; ``gate`` [N, H] logits or None."""
+    window; ``gate`` [N, H] logits or None; ``softcap == 0`` means no cap."""
     if use_hip(q):
         return serving_kernels().paged_attention(q, kpool, vpool, batch.block_tables, batch.cu, batch.start,
                                                  batch.tok_seq, batch.positions, scale, window, keep_first,
-                                                 slopes, gate, batch.num_tiles32)
-    return paged_attention_ref(q, kpool, vpool, batch, scale, window, keep_first, slopes, gate)
+                                                 slopes, gate, batch.num_tiles32, float(softcap), bool(sink))
+    return paged_attention_ref(q, kpool, vpool, batch, scale, window, keep_first, slopes, gate, softcap, sink)
