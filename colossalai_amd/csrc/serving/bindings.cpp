@@ -25,7 +25,15 @@ at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, 
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
-                           int64_t num_tiles);
+                           int64_t num_tiles, double softcap, bool sink);
+at::Tensor silu_mul(at::Tensor packed);
+c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::optional<at::Tensor> b,
+                                       c10::optional<at::Tensor> weight, double eps, at::ScalarType out_dtype);
+std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, at::Tensor correction, int64_t top, int64_t group_count,
+                                           int64_t group_keep, int64_t group_top, double renorm_eps);
+at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at::Tensor ids, at::Tensor weights,
+                           c10::optional<at::Tensor> base);
+at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base);
 
 }  // namespace serving
 }  // namespace cai
@@ -42,5 +50,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("short_conv", &s::short_conv, "short causal depthwise convolution with carried tail");
   m.def("gated_delta_rule", &s::gated_delta_rule, "gated delta rule with per-channel decay, carried state");
   m.def("tied_gate_recurrence", &s::tied_gate_recurrence, "HGRN2-style recurrence, carried state");
-  m.def("paged_attention", &s::paged_attention, "ragged paged attention: window, kept prefix, distance bias, gate");
+  m.def("paged_attention", &s::paged_attention, "ragged paged attention: window, kept prefix, distance bias, gate, soft cap, sink");
+  m.def("silu_mul", &s::silu_mul, "silu(gate) * up of a packed [N, 2F] tensor");
+  m.def("add_rms_norm", &s::add_rms_norm, "residual += a (+ b) in place, then the RMS norm of the sum");
+  m.def("grouped_topk_route", &s::grouped_topk_route, "sigmoid router: correction, group-limited top-k, renormalised");
+  m.def("expert_ffn_gemv", &s::expert_ffn_gemv, "chosen experts' feed-forward of a small step, matrix-vector kernels");
+  m.def("expert_combine", &s::expert_combine, "base + weighted sum of each token's expert outputs, float32");
 }

@@ -1,5 +1,6 @@
 // Element-wise serving kernels: token shift with carried previous row,
-// squared ReLU, logit soft-cap, ragged scatter of keys/values into pages.
+// squared ReLU, gated SiLU of a packed tensor, logit soft-cap, ragged scatter
+// of keys/values into pages.
 #include "serving_common.h"
 
 namespace cai {
@@ -132,6 +133,34 @@ void paged_kv_write(at::Tensor k, at::Tensor v, at::Tensor kpool, at::Tensor vpo
                        rows.data_ptr<int>(), KW, VW);
   });
   HIP_CHECK_LAST();
+}
+
+// packed [N, 2F] = [gate | up], rows strided by ps -> out [N, F] = silu(gate) * up, formed in float32
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ packed, long ps,
+                                                       long N, int F) {
+  const long total = N * F;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long n = i / F;
+    const int f = (int)(i % F);
+    const float g = ldf(packed + n * ps + f), u = ldf(packed + n * ps + F + f);
+    stf(out + i, g * sigmoidf_(g) * u);
+  }
+}
+
+at::Tensor silu_mul(at::Tensor packed) {
+  check_act(packed, "packed");
+  TORCH_CHECK(packed.dim() == 2 && packed.stride(1) == 1 && packed.size(1) % 2 == 0, "packed must be [N, 2F] with dense rows");
+  const long N = packed.size(0);
+  const int F = (int)(packed.size(1) / 2);
+  at::Tensor out = at::empty({N, F}, packed.options());
+  if (N * F == 0) return out;
+  SERVING_DISPATCH_ACT(packed, T, {
+    hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(capped_grid((N * F + 255) / 256, 4096)), dim3(256), 0, stream(),
+                       ptr<T>(out), ptr<T>(packed), (long)packed.stride(0), N, F);
+  });
+  HIP_CHECK_LAST();
+  return out;
 }
 
 }  // namespace serving

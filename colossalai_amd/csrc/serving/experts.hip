@@ -1,0 +1,303 @@
+// Mixture-of-experts serving kernels:
+//   grouped_topk_route : sigmoid scores, a selection-only correction, group-limited
+//                        top-k with ties to the lower index, chosen scores renormalised;
+//   expert_ffn_gemv    : a small step's chosen experts as two matrix-vector kernels
+//                        (up + squared ReLU per (token, expert) pair, then the weighted
+//                        down products of a token summed with its base row) — only the
+//                        chosen experts' weights are streamed, nothing goes to the host;
+//   expert_combine     : base + weighted sum of each token's rows of a sorted-by-expert
+//                        output (the large-step path, whose products are library GEMMs).
+#include "serving_common.h"
+
+namespace cai {
+namespace serving {
+
+// ------------------------------------------------------------------ router
+// One wave per token, four tokens per block; every wave runs every barrier (a wave past the
+// last token repeats the last token and writes nothing). LDS per wave: scores [E], choice
+// scores [E], group worths [groups], picked scores [top].
+__global__ __launch_bounds__(256) void grouped_topk_route_kernel(
+    int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ logits, const float* __restrict__ corr,
+    long N, int E, int top, int groups, int keep, int group_top, float eps) {
+  extern __shared__ float lds[];
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* sc = lds + (long)wid * (2 * E + groups + top);
+  float* ch = sc + E;
+  float* worth = ch + E;
+  float* pick = worth + groups;
+  const long tok = (long)blockIdx.x * 4 + wid;
+  const bool live = tok < N;
+  const long n = live ? tok : N - 1;
+  for (int e = lane; e < E; e += 64) {
+    const float s = sigmoidf_(logits[n * E + e]);
+    sc[e] = s;
+    ch[e] = s + corr[e];
+  }
+  __syncthreads();
+  if (groups > 1) {
+    const int per = E / groups;
+    for (int g = lane; g < groups; g += 64) {
+      // the group_top largest of the group, taken in (value desc, index asc) order
+      float sum = 0.0f, pv = INFINITY;
+      int pi = -1;
+      for (int t = 0; t < group_top && t < per; ++t) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (int k = 0; k < per; ++k) {
+          const float v = ch[g * per + k];
+          const bool after = v < pv || (v == pv && k > pi);   // not yet taken
+          if (after && (bi < 0 || v > bv)) { bv = v; bi = k; }
+        }
+        if (bi < 0) break;
+        sum += bv;
+        pv = bv;
+        pi = bi;
+      }
+      worth[g] = sum;
+    }
+    __syncthreads();
+    for (int g = lane; g < groups; g += 64) {
+      int rank = 0;
+      const float mine = worth[g];
+      for (int o = 0; o < groups; ++o) rank += (worth[o] > mine || (worth[o] == mine && o < g)) ? 1 : 0;
+      if (rank >= keep)
+        for (int k = 0; k < per; ++k) ch[g * per + k] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  float total = 0.0f;
+  for (int t = 0; t < top; ++t) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = ch[e];
+      if (v > bv) { bv = v; bi = e; }   // ascending e: the first of equal values stays
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off);
+      const int oi = __shfl_xor(bi, off);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (bi >= E) bi = 0;  // nothing left to choose from (the host rules this out)
+    if (lane == 0) {
+      pick[t] = sc[bi];
+      ch[bi] = -INFINITY;
+      if (live) ids[tok * top + t] = bi;
+    }
+    total += sc[bi];
+    __syncthreads();
+  }
+  if (live)
+    for (int t = lane; t < top; t += 64) wts[tok * top + t] = pick[t] / (total + eps);
+}
+
+std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, at::Tensor correction, int64_t top, int64_t group_count,
+                                           int64_t group_keep, int64_t group_top, double renorm_eps) {
+  TORCH_CHECK(logits.is_cuda() && is_f32(logits) && logits.dim() == 2 && logits.is_contiguous(),
+              "router logits must be contiguous float32 [N, E]");
+  const long N = logits.size(0);
+  const int E = (int)logits.size(1);
+  TORCH_CHECK(group_count >= 1 && E % group_count == 0 && group_keep >= 1 && group_keep <= group_count && group_top >= 1);
+  TORCH_CHECK(top >= 1 && top <= (E / group_count) * group_keep, "more experts to choose than the kept groups hold");
+  at::Tensor corr = f32c(correction);
+  TORCH_CHECK(corr.numel() == E && corr.is_cuda());
+  at::Tensor ids = at::empty({N, top}, logits.options().dtype(at::kInt));
+  at::Tensor wts = at::empty({N, top}, logits.options());
+  if (N == 0) return {ids, wts};
+  const size_t smem = (size_t)4 * (2 * E + group_count + top) * sizeof(float);
+  TORCH_CHECK(smem <= 64 * 1024, "too many experts for the router kernel");
+  hipLaunchKernelGGL(grouped_topk_route_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), smem, stream(),
+                     ids.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(), corr.data_ptr<float>(), N, E,
+                     (int)top, (int)group_count, (int)group_keep, (int)group_top, (float)renorm_eps);
+  HIP_CHECK_LAST();
+  return {ids, wts};
+}
+
+// ------------------------------------------------------- matrix-vector path
+constexpr int GEMV_R = 4;  // output rows per wave: the input slice a lane holds is reused for each
+
+// dot products of R consecutive rows of `w` (row length K, first row `row0`, `rows` rows exist)
+// with the vector `x`; every lane holds partial sums over its slices of K.
+template <typename T, int R>
+DEV_INLINE void rows_dot(const T* __restrict__ x, const T* __restrict__ w, int K, int row0, int rows, int lane, int vec,
+                         float scale, float* acc) {
+  if (vec) {
+    for (int c = lane * 8; c < K; c += 512) {
+      float xv[8];
+      load8(x + c, xv);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (row0 + r < rows) {
+          float wv[8];
+          load8(w + (long)(row0 + r) * K + c, wv);
+          float d = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) d += xv[i] * wv[i];
+          acc[r] += scale * d;
+        }
+      }
+    }
+  } else {
+    for (int c = lane; c < K; c += 64) {
+      const float xv = ldf(x + c);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (row0 + r < rows) acc[r] += scale * xv * ldf(w + (long)(row0 + r) * K + c);
+    }
+  }
+}
+
+// block = (pair, chunk of 4 * R hidden rows): hidden[p, f] = relu(up_e[f, :] . h[n, :])^2
+template <typename T>
+__global__ __launch_bounds__(256) void expert_up_gemv_kernel(
+    T* __restrict__ hidden, const T* __restrict__ h, const T* __restrict__ w_up, const int* __restrict__ ids, int top,
+    int E, int F, int W, int vec) {
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long p = blockIdx.x;
+  const long n = p / top;
+  const int e = ids[p];
+  const int row0 = (blockIdx.y * 4 + wid) * GEMV_R;
+  if (row0 >= F || e < 0 || e >= E) return;
+  float acc[GEMV_R];
+#pragma unroll
+  for (int r = 0; r < GEMV_R; ++r) acc[r] = 0.0f;
+  rows_dot<T, GEMV_R>(h + n * W, w_up + (long)e * F * W, W, row0, F, lane, vec, 1.0f, acc);
+#pragma unroll
+  for (int r = 0; r < GEMV_R; ++r) {
+    const float v = fmaxf(wave_reduce_sum(acc[r]), 0.0f);
+    if (lane == 0 && row0 + r < F) stf(hidden + p * F + row0 + r, v * v);
+  }
+}
+
+// block = (token, chunk of 4 * R output rows): out[n, w] = base[n, w] + sum_j weight_j down_{e_j}[w, :] . hidden[n, j, :]
+template <typename T, typename TB>
+__global__ __launch_bounds__(256) void expert_down_gemv_kernel(
+    float* __restrict__ out, const T* __restrict__ hidden, const T* __restrict__ w_down, const int* __restrict__ ids,
+    const float* __restrict__ weights, const TB* __restrict__ base, int top, int E, int F, int W, int vec) {
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long n = blockIdx.x;
+  const int row0 = (blockIdx.y * 4 + wid) * GEMV_R;
+  if (row0 >= W) return;
+  float acc[GEMV_R];
+#pragma unroll
+  for (int r = 0; r < GEMV_R; ++r) acc[r] = 0.0f;
+  for (int j = 0; j < top; ++j) {
+    const int e = ids[n * top + j];
+    if (e < 0 || e >= E) continue;
+    rows_dot<T, GEMV_R>(hidden + (n * top + j) * F, w_down + (long)e * W * F, F, row0, W, lane, vec,
+                        weights[n * top + j], acc);
+  }
+#pragma unroll
+  for (int r = 0; r < GEMV_R; ++r) {
+    const float v = wave_reduce_sum(acc[r]);
+    if (lane == 0 && row0 + r < W) {
+      const long at = n * W + row0 + r;
+      out[at] = (base != nullptr ? ldf(base + at) : 0.0f) + v;
+    }
+  }
+}
+
+static void check_experts(const at::Tensor& h, const at::Tensor& w_up, const at::Tensor& w_down, const at::Tensor& ids,
+                          const at::Tensor& weights, const c10::optional<at::Tensor>& base) {
+  check_act(h, "h");
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous(), "h must be contiguous [N, W]");
+  TORCH_CHECK(w_up.dim() == 3 && w_down.dim() == 3 && w_up.is_contiguous() && w_down.is_contiguous() && w_up.is_cuda() &&
+              w_down.is_cuda(), "expert matrices must be contiguous [E, out, in] GPU tensors");
+  TORCH_CHECK(w_up.scalar_type() == h.scalar_type() && w_down.scalar_type() == h.scalar_type(),
+              "experts and their input share one dtype");
+  TORCH_CHECK(w_up.size(2) == h.size(1) && w_down.size(0) == w_up.size(0) && w_down.size(1) == h.size(1) &&
+              w_down.size(2) == w_up.size(1), "expert matrix shapes do not fit [E, F, W] / [E, W, F]");
+  check_i32(ids, "ids");
+  TORCH_CHECK(ids.dim() == 2 && ids.size(0) == h.size(0));
+  TORCH_CHECK(weights.is_cuda() && is_f32(weights) && weights.is_contiguous() && weights.sizes() == ids.sizes(),
+              "weights must be contiguous float32 of the ids' shape");
+  if (base.has_value()) {
+    check_act(*base, "base");
+    TORCH_CHECK(base->is_contiguous() && base->sizes() == h.sizes(), "base must be contiguous and of h's shape");
+  }
+}
+
+at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at::Tensor ids, at::Tensor weights,
+                           c10::optional<at::Tensor> base) {
+  check_experts(h, w_up, w_down, ids, weights, base);
+  const long N = h.size(0);
+  const int W = (int)h.size(1), E = (int)w_up.size(0), F = (int)w_up.size(1), top = (int)ids.size(1);
+  at::Tensor out = at::empty({N, W}, h.options().dtype(at::kFloat));
+  if (N == 0) return out;
+  at::Tensor hidden = at::empty({N * top, F}, h.options());
+  const int rows_per_block = 4 * GEMV_R;
+  // 8-element slices need rows that start 16 bytes (bfloat16) / 32 bytes (float32) apart
+  auto aligned = [](const at::Tensor& t) { return reinterpret_cast<uintptr_t>(t.data_ptr()) % 32 == 0; };
+  const int vec_up = (W % 8 == 0 && aligned(h) && aligned(w_up)) ? 1 : 0;
+  const int vec_down = (F % 8 == 0 && aligned(hidden) && aligned(w_down)) ? 1 : 0;
+  SERVING_DISPATCH_ACT(h, T, {
+    hipLaunchKernelGGL(expert_up_gemv_kernel<T>, dim3((unsigned)(N * top), (unsigned)((F + rows_per_block - 1) / rows_per_block)),
+                       dim3(256), 0, stream(), ptr<T>(hidden), ptr<T>(h), ptr<T>(w_up), ids.data_ptr<int>(), top, E, F, W,
+                       vec_up);
+    const dim3 grid((unsigned)N, (unsigned)((W + rows_per_block - 1) / rows_per_block));
+    if (base.has_value()) {
+      SERVING_DISPATCH_ACT(*base, TB, {
+        hipLaunchKernelGGL((expert_down_gemv_kernel<T, TB>), grid, dim3(256), 0, stream(), out.data_ptr<float>(),
+                           ptr<T>(hidden), ptr<T>(w_down), ids.data_ptr<int>(), weights.data_ptr<float>(), ptr<TB>(*base),
+                           top, E, F, W, vec_down);
+      });
+    } else {
+      hipLaunchKernelGGL((expert_down_gemv_kernel<T, float>), grid, dim3(256), 0, stream(), out.data_ptr<float>(),
+                         ptr<T>(hidden), ptr<T>(w_down), ids.data_ptr<int>(), weights.data_ptr<float>(),
+                         (const float*)nullptr, top, E, F, W, vec_down);
+    }
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
+// ------------------------------------------------------------------ combine
+// out[n, w] = base[n, w] + sum_j weights[n, j] * y[inv[n, j], w], slots in order, float32
+template <typename T, typename TB>
+__global__ __launch_bounds__(256) void expert_combine_kernel(
+    float* __restrict__ out, const T* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
+    const TB* __restrict__ base, int top, int W, long rows) {
+  const long n = blockIdx.x;
+  for (int w = threadIdx.x; w < W; w += blockDim.x) {
+    float acc = base != nullptr ? ldf(base + n * W + w) : 0.0f;
+    for (int j = 0; j < top; ++j) {
+      const long r = inv[n * top + j];
+      if (r >= 0 && r < rows) acc += weights[n * top + j] * ldf(y + r * W + w);
+    }
+    out[n * W + w] = acc;
+  }
+}
+
+at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base) {
+  check_act(y, "y");
+  check_i32(inv, "inv");
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && inv.dim() == 2 && inv.size(0) * inv.size(1) == y.size(0),
+              "y must be contiguous [N * top, W] and inv [N, top]");
+  TORCH_CHECK(weights.is_cuda() && is_f32(weights) && weights.is_contiguous() && weights.sizes() == inv.sizes());
+  const long N = inv.size(0);
+  const int top = (int)inv.size(1), W = (int)y.size(1);
+  if (base.has_value()) {
+    check_act(*base, "base");
+    TORCH_CHECK(base->is_contiguous() && base->dim() == 2 && base->size(0) == N && base->size(1) == W);
+  }
+  at::Tensor out = at::empty({N, W}, y.options().dtype(at::kFloat));
+  if (N == 0) return out;
+  SERVING_DISPATCH_ACT(y, T, {
+    if (base.has_value()) {
+      SERVING_DISPATCH_ACT(*base, TB, {
+        hipLaunchKernelGGL((expert_combine_kernel<T, TB>), dim3((unsigned)N), dim3(256), 0, stream(), out.data_ptr<float>(),
+                           ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), ptr<TB>(*base), top, W, (long)y.size(0));
+      });
+    } else {
+      hipLaunchKernelGGL((expert_combine_kernel<T, float>), dim3((unsigned)N), dim3(256), 0, stream(), out.data_ptr<float>(),
+                         ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), (const float*)nullptr, top, W,
+                         (long)y.size(0));
+    }
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
+}  // namespace serving
+}  // namespace cai

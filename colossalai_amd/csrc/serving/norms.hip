@@ -5,7 +5,10 @@
 //                        weight and an optional sigmoid gate;
 //   merge_rms_norm     : two branch rows, each full-width RMS-normed with its
 //                        own weight, averaged, group-normed and added to the
-//                        residual — one pass, the merged row staged in LDS.
+//                        residual — one pass, the merged row staged in LDS;
+//   add_rms_norm       : residual += a (+ b) in place and, when a weight is
+//                        given, the RMS norm of the new residual row for the
+//                        next pre-norm layer, in one launch.
 #include "serving_common.h"
 
 namespace cai {
@@ -190,6 +193,73 @@ at::Tensor merge_rms_norm(at::Tensor a, at::Tensor wa, at::Tensor b, at::Tensor 
   });
   HIP_CHECK_LAST();
   return residual;
+}
+
+// One block per row. Pass 1 forms r = residual + (a + b) in float32, stores it and sums r^2; pass 2
+// (only with a weight) re-reads the elements this same thread stored and writes the normed row.
+template <typename TA, typename TB, typename TO>
+__global__ __launch_bounds__(256) void add_rms_norm_kernel(
+    TO* __restrict__ out, float* __restrict__ residual, const TA* __restrict__ a, const TB* __restrict__ b,
+    const float* __restrict__ w, int W, float eps) {
+  __shared__ float red[8];
+  const long row = blockIdx.x;
+  float* rr = residual + row * W;
+  float ssq = 0.0f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float add = ldf(a + row * W + i);
+    if (b != nullptr) add += ldf(b + row * W + i);
+    const float r = rr[i] + add;
+    rr[i] = r;
+    ssq += r * r;
+  }
+  if (w == nullptr) return;
+  ssq = block_reduce_sum(ssq, red);
+  const float inv = 1.0f / sqrtf(ssq / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + row * W + i, rr[i] * inv * w[i]);
+}
+
+c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::optional<at::Tensor> b,
+                                       c10::optional<at::Tensor> weight, double eps, at::ScalarType out_dtype) {
+  check_act(a, "a");
+  TORCH_CHECK(residual.is_cuda() && is_f32(residual) && residual.dim() == 2 && residual.is_contiguous(),
+              "residual must be contiguous float32 [N, W]");
+  TORCH_CHECK(a.is_contiguous() && a.sizes() == residual.sizes(), "a must be contiguous and of the residual's shape");
+  if (b.has_value()) {
+    check_act(*b, "b");
+    TORCH_CHECK(b->is_contiguous() && b->sizes() == residual.sizes(), "b must be contiguous and of the residual's shape");
+  }
+  const long N = residual.size(0);
+  const int W = (int)residual.size(1);
+  at::Tensor w, out;
+  const float* wp = nullptr;
+  if (weight.has_value()) {
+    w = f32c(*weight);
+    TORCH_CHECK(w.numel() == W);
+    wp = w.data_ptr<float>();
+    out = at::empty({N, W}, residual.options().dtype(out_dtype));
+    check_act(out, "out");
+  }
+  if (N > 0) {
+    // without a weight nothing is written through `out`: any instantiation of TO will do
+    const at::Tensor& like = weight.has_value() ? out : residual;
+    SERVING_DISPATCH_ACT(a, TA, {
+      SERVING_DISPATCH_ACT(like, TO, {
+        TO* op = weight.has_value() ? ptr<TO>(out) : (TO*)nullptr;
+        if (b.has_value()) {
+          SERVING_DISPATCH_ACT(*b, TB, {
+            hipLaunchKernelGGL((add_rms_norm_kernel<TA, TB, TO>), dim3((unsigned)N), dim3(256), 0, stream(), op,
+                               residual.data_ptr<float>(), ptr<TA>(a), ptr<TB>(*b), wp, W, (float)eps);
+          });
+        } else {
+          hipLaunchKernelGGL((add_rms_norm_kernel<TA, float, TO>), dim3((unsigned)N), dim3(256), 0, stream(), op,
+                             residual.data_ptr<float>(), ptr<TA>(a), (const float*)nullptr, wp, W, (float)eps);
+        }
+      });
+    });
+    HIP_CHECK_LAST();
+  }
+  if (!weight.has_value()) return c10::nullopt;
+  return out;
 }
 
 }  // namespace serving

@@ -1,5 +1,7 @@
 // Attention of a ragged batch over paged keys/values with a sliding window,
-// kept first tokens, a linear distance penalty and a per-head output gate.
+// kept first tokens, a linear distance penalty, a per-head output gate, a tanh
+// soft cap on the scaled score and an optional sink (one more place of score 0
+// in the softmax denominator that carries no value).
 //
 // One wave per (token, query head). The visible keys of a token are two
 // position ranges: the kept prefix [0, min(keep_first, lo)) and the window
@@ -26,26 +28,6 @@ DEV_INLINE float dpp_add(float v) {
 // sum over the 8 adjacent lanes that share a key (quad xor 1, quad xor 2, half-row mirror)
 DEV_INLINE float reduce8(float v) { return dpp_add<0x141>(dpp_add<0x4E>(dpp_add<0xB1>(v))); }
 
-// 8 consecutive elements of a key row as floats
-DEV_INLINE void load8(const float* p, float* o) {
-  const float4v a = *reinterpret_cast<const float4v*>(p), b = *reinterpret_cast<const float4v*>(p + 4);
-  o[0] = a[0]; o[1] = a[1]; o[2] = a[2]; o[3] = a[3]; o[4] = b[0]; o[5] = b[1]; o[6] = b[2]; o[7] = b[3];
-}
-DEV_INLINE void load8(const bf16s* p, float* o) {
-  const short8 a = *reinterpret_cast<const short8*>(p);
-#pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = bf2f((bf16s)a[e]);
-}
-// two consecutive value channels
-DEV_INLINE void load2(const float* p, float& a, float& b) {
-  const float2v t = *reinterpret_cast<const float2v*>(p);
-  a = t[0]; b = t[1];
-}
-DEV_INLINE void load2(const bf16s* p, float& a, float& b) {
-  const unsigned int t = *reinterpret_cast<const unsigned int*>(p);
-  a = bf2f((bf16s)(t & 0xffffu)); b = bf2f((bf16s)(t >> 16));
-}
-
 // Scalar kernel (decode tokens, float32 serving, shapes the MFMA kernel does not take).
 // One block per (token, kv head, group of up to RC query heads of that kv head): keys and
 // values are read once for the whole group. The block's nw waves (16, or 8 when the partial
@@ -62,7 +44,8 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, const float* __restrict__ slopes, const T* __restrict__ gate, long gate_stride,
-    int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec, int vvec) {
+    int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec, int vvec,
+    float softcap, int sink) {
   extern __shared__ __align__(16) float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const int Dp = (D + 7) & ~7;
@@ -92,6 +75,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int n_keep = window > 0 ? min(keep_first, lo) : 0;
   const int total = n_keep + (pos - lo + 1);
+  const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
   const int part8 = lane & 7, ksub = lane >> 3;
   const int DS = (((D + 7) >> 3) + 7) & ~7;  // slice of the head size per lane, a multiple of 8
   const int d_lo = part8 * DS, d_hi = min(D, d_lo + DS);
@@ -139,8 +123,11 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
       for (int r = 0; r < RC; ++r) dots[r] = reduce8(dots[r]);
       if (part8 == 0) {
 #pragma unroll
-        for (int r = 0; r < RC; ++r)
-          pw[r * 64 + sub * 8 + ksub] = valid ? dots[r] * scale - slope[r] * (float)(pos - j) : -INFINITY;
+        for (int r = 0; r < RC; ++r) {
+          float sc = dots[r] * scale;
+          if (softcap > 0.0f) sc = softcap * tanhf(sc * inv_cap);
+          pw[r * 64 + sub * 8 + ksub] = valid ? sc - slope[r] * (float)(pos - j) : -INFINITY;
+        }
         prow[sub * 8 + ksub] = row;
       }
     };
@@ -215,6 +202,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
         o += part[(w * RC + r) * PS + 2 + dv] * f;
       }
     }
+    if (sink) ll += expf(-mm);  // the sink's score is 0
     float scale_out = 1.0f / ll;
     if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h0 + r));
     stf(out + (n * H + h0 + r) * (long)Dv + dv, o * scale_out);
@@ -238,7 +226,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     bf16s* __restrict__ out, const bf16s* __restrict__ q, long q_stride, const bf16s* __restrict__ kpool,
     const bf16s* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu,
     const int* __restrict__ start, const float* __restrict__ slopes, const bf16s* __restrict__ gate, long gate_stride,
-    int H, int G, int page_shift, float scale, int window, int keep_first) {
+    int H, int G, int page_shift, float scale, int window, int keep_first, float softcap, int sink) {
   constexpr int D = DS * 16, Dv = VT * 32;
   constexpr int KP = D + 8;            // key row pitch in LDS (elements): 16-byte reads of 16 rows hit 64 banks
   constexpr int VP = 40;               // transposed value row pitch: 32 key slots + 8
@@ -335,6 +323,14 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     for (int i = 0; i < 16; ++i) oacc[t][i] = 0.0f;
   constexpr float LOG2E = 1.4426950408889634f;
   const float c1 = scale * LOG2E, sl2 = slope * LOG2E;
+  // soft cap in the base-2 domain: cap log2e tanh(x scale / cap), tanh(y) = 1 - 2 / (exp2(2 log2e y) + 1)
+  const bool capped = softcap > 0.0f;
+  const float cap2 = softcap * LOG2E, t2 = capped ? 2.0f * LOG2E * scale / softcap : 0.0f;
+  auto base2 = [&](float dot) {
+    if (!capped) return dot * c1;
+    const float e = __builtin_amdgcn_exp2f(fminf(dot * t2, 64.0f));  // beyond 2^64 the quotient is 0 in float32 anyway
+    return cap2 - 2.0f * cap2 * __builtin_amdgcn_rcpf(e + 1.0f);
+  };
   float row_bias[16];  // + slope log2e * (row of the C layout): the key's offset inside its tile
 #pragma unroll
   for (int i = 0; i < 16; ++i) row_bias[i] = sl2 * (float)((i & 3) + 8 * (i >> 2) + 4 * hf);
@@ -369,7 +365,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       if (interior) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          sv[i] = sacc[i] * c1 + (tile_bias + row_bias[i]);
+          sv[i] = base2(sacc[i]) + (tile_bias + row_bias[i]);
           tmax = fmaxf(tmax, sv[i]);
         }
       } else {
@@ -377,7 +373,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         for (int i = 0; i < 16; ++i) {
           const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
           const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
-          sv[i] = seen ? sacc[i] * c1 + (tile_bias + row_bias[i]) : -INFINITY;
+          sv[i] = seen ? base2(sacc[i]) + (tile_bias + row_bias[i]) : -INFINITY;
           tmax = fmaxf(tmax, sv[i]);
         }
       }
@@ -417,6 +413,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     __syncthreads();
   }
   l += __shfl_xor(l, 32);
+  if (sink) l += __builtin_amdgcn_exp2f(-m);  // the sink's score is 0 in either base; m is finite (a token sees itself)
   if (!tok_ok || !head_ok) return;
   float scale_out = 1.0f / l;
   if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h));
@@ -435,8 +432,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
-                           int64_t num_tiles) {
+                           int64_t num_tiles, double softcap, bool sink) {
   check_act(q, "q");
+  TORCH_CHECK(softcap >= 0.0, "softcap must not be negative (0 = none)");
   TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1 && q.stride(1) == q.size(2), "q must be [N, H, D] with dense rows");
   TORCH_CHECK(kpool.dim() == 4 && vpool.dim() == 4 && kpool.is_contiguous() && vpool.is_contiguous());
   TORCH_CHECK(kpool.scalar_type() == q.scalar_type() && vpool.scalar_type() == q.scalar_type(),
@@ -480,7 +478,8 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
                      ptr<bf16s>(q), (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool),                        \
                      block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu.data_ptr<int>(),                 \
                      start.data_ptr<int>(), slp, gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr,      \
-                     gstride, H, G, page_shift, (float)scale, (int)window, (int)keep_first)
+                     gstride, H, G, page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap,     \
+                     sink ? 1 : 0)
     if (D == 32) MFMA_CASE(2, 1);
     else if (D == 64 && Dv == 64) MFMA_CASE(4, 2);
     else if (D == 64 && Dv == 128) MFMA_CASE(4, 4);
@@ -506,7 +505,8 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
                      stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),             \
                      block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),            \
                      positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride, \
-                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec)
+                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec,                \
+                     (float)softcap, sink ? 1 : 0)
   SERVING_DISPATCH_ACT(q, T, {
     if (rc == 4) SCALAR_CASE(4);
     else if (rc == 2) SCALAR_CASE(2);

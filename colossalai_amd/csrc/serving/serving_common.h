@@ -24,6 +24,26 @@ DEV_INLINE void stf(bf16s* p, float v) { *p = f2bf(v); }
 DEV_INLINE float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 DEV_INLINE float softplusf_(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
 
+// 8 consecutive elements of a row as floats (16-byte aligned for bf16, 32-byte for float)
+DEV_INLINE void load8(const float* p, float* o) {
+  const float4v a = *reinterpret_cast<const float4v*>(p), b = *reinterpret_cast<const float4v*>(p + 4);
+  o[0] = a[0]; o[1] = a[1]; o[2] = a[2]; o[3] = a[3]; o[4] = b[0]; o[5] = b[1]; o[6] = b[2]; o[7] = b[3];
+}
+DEV_INLINE void load8(const bf16s* p, float* o) {
+  const short8 a = *reinterpret_cast<const short8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = bf2f((bf16s)a[e]);
+}
+// two consecutive elements
+DEV_INLINE void load2(const float* p, float& a, float& b) {
+  const float2v t = *reinterpret_cast<const float2v*>(p);
+  a = t[0]; b = t[1];
+}
+DEV_INLINE void load2(const bf16s* p, float& a, float& b) {
+  const unsigned int t = *reinterpret_cast<const unsigned int*>(p);
+  a = bf2f((bf16s)(t & 0xffffu)); b = bf2f((bf16s)(t >> 16));
+}
+
 inline hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
 
 inline bool is_bf16(const at::Tensor& t) { return t.scalar_type() == at::kBFloat16; }
