@@ -221,13 +221,19 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
 //                  order, one 16-byte read per product)
 // so column = token = lane & 31 everywhere: running max, running sum, rescaling and the gate
 // never cross lanes except for one exchange between the two half-waves.
+// The tiles are DS * 16 key channels by VT * 32 value channels; a head whose sizes Dr / Dvr are
+// smaller (multiples of 8) is padded with zeros on its way into registers and LDS, and only its
+// own channels are stored.
 template <int DS, int VT>
 __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     bf16s* __restrict__ out, const bf16s* __restrict__ q, long q_stride, const bf16s* __restrict__ kpool,
     const bf16s* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu,
     const int* __restrict__ start, const float* __restrict__ slopes, const bf16s* __restrict__ gate, long gate_stride,
-    int H, int G, int page_shift, float scale, int window, int keep_first, float softcap, int sink) {
+    int H, int G, int Dr, int Dvr, int page_shift, float scale, int window, int keep_first, float softcap, int sink) {
   constexpr int D = DS * 16, Dv = VT * 32;
+  bf16x8_v zero8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zero8[e] = (__bf16)0.0f;
   constexpr int KP = D + 8;            // key row pitch in LDS (elements): 16-byte reads of 16 rows hit 64 banks
   constexpr int VP = 40;               // transposed value row pitch: 32 key slots + 8
   constexpr int KT = 32 * KP, VTT = Dv * VP;   // elements of one staged tile
@@ -261,7 +267,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 
   bf16x8_v qf[DS];
 #pragma unroll
-  for (int s = 0; s < DS; ++s) qf[s] = ld_g16b(q + n * q_stride + (long)h * D + 16 * s + hf * 8);
+  for (int s = 0; s < DS; ++s)
+    qf[s] = 16 * s + hf * 8 < Dr ? ld_g16b(q + n * q_stride + (long)h * Dr + 16 * s + hf * 8) : zero8;
 
   const int lo_min = window > 0 ? max(0, p0 - window + 1) : 0;
   const int wstart = lo_min & ~31;
@@ -282,12 +289,18 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
       const int c = tid + nthreads * r;
-      if (c < KCH) rk[r] = ld_g16b(kpool + (pool_row(kbase + c / (D / 8)) * G + g) * D + 8 * (c % (D / 8)));
+      if (c < KCH) {
+        const int off = 8 * (c % (D / 8));
+        rk[r] = off < Dr ? ld_g16b(kpool + (pool_row(kbase + c / (D / 8)) * G + g) * Dr + off) : zero8;
+      }
     }
 #pragma unroll
     for (int r = 0; r < VR; ++r) {
       const int c = tid + nthreads * r;
-      if (c < VCH) rv[r] = ld_g16b(vpool + (pool_row(kbase + c / (Dv / 8)) * G + g) * Dv + 8 * (c % (Dv / 8)));
+      if (c < VCH) {
+        const int off = 8 * (c % (Dv / 8));
+        rv[r] = off < Dvr ? ld_g16b(vpool + (pool_row(kbase + c / (Dv / 8)) * G + g) * Dvr + off) : zero8;
+      }
     }
   };
   auto stash = [&](int buf) {
@@ -417,11 +430,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   if (!tok_ok || !head_ok) return;
   float scale_out = 1.0f / l;
   if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h));
-  bf16s* orow = out + (n * H + h) * (long)Dv;
+  bf16s* orow = out + (n * H + h) * (long)Dvr;
 #pragma unroll
   for (int t = 0; t < VT; ++t)
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
+      if (t * 32 + 8 * a + 4 * hf >= Dvr) continue;  // padding channels (sizes are multiples of 8: four at a time)
       short4v pk;
 #pragma unroll
       for (int c = 0; c < 4; ++c) pk[c] = (short)f2bf(oacc[t][4 * a + c] * scale_out);
@@ -468,23 +482,33 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   // prompt portions in bfloat16 go to the matrix cores when the head sizes fit a tiling;
   // num_tiles = sum over sequences of ceil(new tokens / 32), 0 asks for the scalar kernel
   const bool aligned = q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0;
-  const bool mfma_shape = (D == 32 && Dv == 32) || ((D == 64 || D == 128) && (Dv == 64 || Dv == 128));
+  // head sizes that are multiples of 8 ride in the next larger tiling, zero-padded
+  const bool mfma_shape = D % 8 == 0 && Dv % 8 == 0 && D <= 128 && Dv <= 128;
   if (num_tiles > 0 && is_bf16(q) && aligned && mfma_shape) {
     const int rep = H / G, nw = 4;
     const dim3 grid((unsigned)num_tiles, (unsigned)G, (unsigned)((rep + nw - 1) / nw));
-    const size_t msmem = (size_t)2 * (32 * (D + 8) + Dv * 40) * sizeof(bf16s);
+    const int ds = D <= 32 ? 2 : D <= 48 ? 3 : D <= 64 ? 4 : D <= 96 ? 6 : 8, vt = (Dv + 31) / 32;
+    const size_t msmem = (size_t)2 * (32 * (ds * 16 + 8) + vt * 32 * 40) * sizeof(bf16s);
 #define MFMA_CASE(DS_, VT_)                                                                                          \
   hipLaunchKernelGGL((paged_attention_mfma_kernel<DS_, VT_>), grid, dim3(64 * nw), msmem, stream(), ptr<bf16s>(out), \
                      ptr<bf16s>(q), (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool),                        \
                      block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu.data_ptr<int>(),                 \
                      start.data_ptr<int>(), slp, gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr,      \
-                     gstride, H, G, page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap,     \
+                     gstride, H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap,     \
                      sink ? 1 : 0)
-    if (D == 32) MFMA_CASE(2, 1);
-    else if (D == 64 && Dv == 64) MFMA_CASE(4, 2);
-    else if (D == 64 && Dv == 128) MFMA_CASE(4, 4);
-    else if (D == 128 && Dv == 64) MFMA_CASE(8, 2);
-    else MFMA_CASE(8, 4);
+#define MFMA_ROW(DS_)                     \
+  do {                                    \
+    if (vt == 1) MFMA_CASE(DS_, 1);       \
+    else if (vt == 2) MFMA_CASE(DS_, 2);  \
+    else if (vt == 3) MFMA_CASE(DS_, 3);  \
+    else MFMA_CASE(DS_, 4);               \
+  } while (0)
+    if (ds == 2) MFMA_ROW(2);
+    else if (ds == 3) MFMA_ROW(3);
+    else if (ds == 4) MFMA_ROW(4);
+    else if (ds == 6) MFMA_ROW(6);
+    else MFMA_ROW(8);
+#undef MFMA_ROW
 #undef MFMA_CASE
     HIP_CHECK_LAST();
     return out;

@@ -40,13 +40,12 @@ def sink_softcap_attention(q, k, v, scale, softcap):
     for h in range(H):
         g = h // (H // G)
         for i in range(T):
-            s = torch.stack([(q[i, h] * k[j, g]).sum() * scale for j in range(i + 1)])
+            s = (k[: i + 1, g] @ q[i, h]) * scale       # keys 0..i and no others
             if softcap:
                 s = softcap * torch.tanh(s / softcap)
             e = torch.exp(s)
             p = e / (1.0 + e.sum())
-            for j in range(i + 1):
-                out[i, h] += p[j] * v[j, g]
+            out[i, h] = p @ v[: i + 1, g]
     return out
 
 

@@ -5,8 +5,8 @@ continued sequences and single decode tokens, in bfloat16 and float32."""
 import pytest
 import torch
 
-from colossalai_amd.ops import group_norm, linear_recurrence, paged_attention, short_conv, token_shift
-from colossalai_amd.ops.activation import relu_squared, softcap
+from colossalai_amd.ops import group_norm, linear_recurrence, paged_attention, routed_experts, short_conv, token_shift
+from colossalai_amd.ops.activation import relu_squared, silu_mul, softcap
 from colossalai_amd.ops.ragged import RaggedBatch
 
 pytestmark = pytest.mark.gpu
@@ -214,3 +214,108 @@ def test_paged_attention_heads_per_block(counts):
     out = paged_attention.paged_attention(q.cuda(), kpool.cuda(), vpool.cuda(), gb, 0.3, 50, 3, slopes.cuda(), None)
     ref = paged_attention.paged_attention_ref(q, kpool, vpool, cb, 0.3, 50, 3, slopes, None)
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [16, 64])
+@pytest.mark.parametrize("H,G,D,Dv,cap", [(6, 2, 48, 96, 8.0), (4, 2, 40, 80, 0.0), (2, 1, 96, 72, 3.0), (8, 2, 64, 64, 50.0),
+                                          (3, 3, 24, 44, 5.0), (4, 4, 128, 128, 30.0), (4, 2, 16, 8, 1.0),
+                                          (2, 2, 104, 120, 12.0)])
+def test_paged_attention_softcap_and_sink(dtype, H, G, D, Dv, cap, page):
+    """Soft-capped scores and the sink's place in the denominator, in the scalar
+    kernel and in the matrix-core kernel (bfloat16; head sizes that are
+    multiples of 8 ride zero-padded in the next larger tiling)."""
+    torch.manual_seed(9)
+    gb, cb, pages = make_batch("cuda", page)
+    N = gb.num_tokens
+    kpool, vpool = (torch.randn(pages, page, G, D) * 3).to(dtype), (torch.randn(pages, page, G, Dv) * 50).to(dtype)
+    kg, vg = kpool.cuda(), vpool.cuda()
+    q, k, v = torch.randn(N, H, D).to(dtype), torch.randn(N, G, D).to(dtype), torch.randn(N, G, Dv).to(dtype)
+    paged_attention.paged_kv_write(k.cuda(), v.cuda(), kg, vg, gb)
+    paged_attention.paged_kv_write(k, v, kpool, vpool, cb)
+    loose = dict(rtol=2e-2, atol=0.5) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=2e-3)
+    for sink in (True, False):
+        out = paged_attention.paged_attention(q.cuda(), kg, vg, gb, 0.3, softcap=cap, sink=sink)
+        ref = paged_attention.paged_attention_ref(q, kpool, vpool, cb, 0.3, softcap=cap, sink=sink)
+        torch.testing.assert_close(out.cpu().float(), ref.float(), **loose)
+    # decode-only step: the scalar kernel on the same pages
+    tabs = [t.tolist() for t in gb.block_tables[:3]]
+    dec = RaggedBatch.build([1] * 3, [36, 25, 63], [3, 0, 5], "cuda", tabs, page)
+    dec_c = RaggedBatch.build([1] * 3, [36, 25, 63], [3, 0, 5], "cpu", tabs, page)
+    qd = q[[36, 41, 42]]
+    one = paged_attention.paged_attention(qd.cuda(), kg, vg, dec, 0.3, softcap=cap, sink=True)
+    torch.testing.assert_close(one.cpu().float(),
+                               paged_attention.paged_attention_ref(qd, kpool, vpool, dec_c, 0.3, softcap=cap, sink=True).float(),
+                               **loose)
+
+
+def test_sink_with_tiny_scores_halves_nothing_by_accident():
+    """Scores of exactly 0 for t visible keys: every weight is 1 / (t + 1)."""
+    page, T, D, Dv = 16, 40, 32, 32
+    b = RaggedBatch.build([T], [0], [0], "cuda", [[2, 0, 1]], page)
+    kpool = torch.zeros(3, page, 1, D, dtype=torch.bfloat16, device="cuda")
+    vpool = torch.ones(3, page, 1, Dv, dtype=torch.bfloat16, device="cuda")
+    q = torch.randn(T, 2, D, dtype=torch.bfloat16, device="cuda")
+    out = paged_attention.paged_attention(q, kpool, vpool, b, 1.0, softcap=7.0, sink=True).float().cpu()
+    want = torch.arange(1, T + 1).float() / torch.arange(2, T + 2).float()
+    torch.testing.assert_close(out[:, 0, 0], want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("W", [96, 1000])
+def test_add_rms_norm(dtype, W):
+    torch.manual_seed(10)
+    x, w = torch.randn(19, W) * 4, torch.randn(W)
+    a, b = torch.randn(19, W).to(dtype), torch.randn(19, W)  # the second addend may be float32
+    rg, rc = x.clone().cuda(), x.clone()
+    hg = group_norm.add_rms_norm(rg, a.cuda(), b.cuda(), w.cuda(), 1e-5, dtype)
+    hc = group_norm.add_rms_norm_ref(rc, a, b, w, 1e-5, dtype)
+    torch.testing.assert_close(rg.cpu(), rc, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(hg.cpu().float(), hc.float(), **tol(dtype))
+    rg2, rc2 = x.clone().cuda(), x.clone()
+    assert group_norm.add_rms_norm(rg2, a.cuda(), None, None, 1e-5) is None
+    group_norm.add_rms_norm_ref(rc2, a, None, None, 1e-5)
+    torch.testing.assert_close(rg2.cpu(), rc2, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    torch.manual_seed(11)
+    y = (torch.randn(33, 2 * 150 + 10) * 3).to(dtype)
+    out = silu_mul(y.cuda()[:, 10:])
+    g, u = y[:, 10:160].float(), y[:, 160:].float()
+    torch.testing.assert_close(out.cpu().float(), (g * torch.sigmoid(g) * u).to(dtype).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("E,top,groups,keep", [(12, 2, 3, 2), (64, 6, 8, 3), (256, 8, 8, 4), (7, 3, 1, 1), (9, 2, 9, 5),
+                                               (160, 6, 1, 1)])
+def test_grouped_topk_route(E, top, groups, keep):
+    torch.manual_seed(12)
+    z = torch.randn(301, E) * 2
+    corr = torch.randn(E) * 0.4
+    ids, w = routed_experts.grouped_topk_route(z.cuda(), corr.cuda(), top, groups, keep, 2, 1e-20)
+    ids_r, w_r = routed_experts.grouped_topk_route_ref(z, corr, top, groups, keep, 2, 1e-20)
+    same = (ids.cpu() == ids_r).all(-1)
+    assert same.float().mean().item() > 0.99  # a sigmoid that differs in its last bit may swap a near-tie
+    torch.testing.assert_close(w.cpu()[same], w_r[same], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,W,Fe,E,top,shared", [(7, 256, 96, 8, 2, True), (3, 100, 36, 5, 3, False), (1, 512, 200, 4, 4, True),
+                                               (300, 256, 128, 6, 2, True), (200, 96, 40, 16, 1, False)])
+def test_routed_expert_ffn(dtype, N, W, Fe, E, top, shared):
+    """Few pairs: matrix-vector kernels; many: sorted per-expert products and the combine kernel."""
+    torch.manual_seed(13)
+    h = torch.randn(N, W).to(dtype)
+    w_up = (torch.randn(E, Fe, W) / W ** 0.5).to(dtype)
+    w_down = (torch.randn(E, W, Fe) / Fe ** 0.5).to(dtype)
+    ids = torch.stack([torch.randperm(E)[:top] for _ in range(N)]).int()
+    wts = torch.rand(N, top)
+    base = torch.randn(N, W).to(dtype) if shared else None
+    out = routed_experts.routed_expert_ffn(h.cuda(), w_up.cuda(), w_down.cuda(), ids.cuda(), wts.cuda(),
+                                           None if base is None else base.cuda())
+    ref = routed_experts.routed_expert_ffn_ref(h.float(), w_up.float(), w_down.float(), ids, wts,
+                                               None if base is None else base.float())
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.cpu(), ref, **(dict(rtol=3e-2, atol=3e-2) if dtype == torch.bfloat16
+                                                  else dict(rtol=1e-4, atol=1e-4)))
