@@ -29,9 +29,10 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=5)
     p.add_argument("--warmup", type=int, default=2)
-    p.add_argument("--workload", type=str, default="train", choices=["train", "serve-hybrid"],
-                   help="train: the headline training step (default). serve-hybrid: prefill/decode tokens/s of the "
-                        "Kipirax hybrid next to a Llama of equal size, both through the continuous-batching engine")
+    p.add_argument("--workload", type=str, default="train", choices=["train", "serve-hybrid", "serve-moe"],
+                   help="train: the headline training step (default). serve-hybrid / serve-moe: prefill/decode tokens/s "
+                        "of the Kipirax hybrid / the Mubutar routed-experts model next to a Llama of equal size, both "
+                        "through the continuous-batching engine")
     p.add_argument("--serve-sizes", type=str, default="w2048,w4096")
     p.add_argument("--model", type=str, default="llama-7b")
     p.add_argument("--batch", type=int, default=36, help="per-DP-rank batch size (reference: bs/DP=36)")
@@ -50,25 +51,25 @@ def parse_args():
     return p.parse_args()
 
 
-def serve_hybrid(args):
-    """Side workload: serving throughput of the hybrid model beside Llama (one GPU)."""
+def serve_comparison(args, kind):
+    """Side workload: serving throughput of a ragged-step model beside Llama (one GPU)."""
     from colossalai_amd.inference.bench_serving import run_serving_comparison
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py requires an MI355X GPU")
-    res = run_serving_comparison(args.serve_sizes.split(","))
+    res = run_serving_comparison(args.serve_sizes.split(","), kind=kind)
     first = res[args.serve_sizes.split(",")[0]]
     print(json.dumps({
-        "metric": "hybrid_serving_decode_tokens_per_s", "value": round(first["hybrid"]["decode_tok_s"], 1),
+        "metric": f"{kind}_serving_decode_tokens_per_s", "value": round(first[kind]["decode_tok_s"], 1),
         "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
-        "vs_baseline": None, "config": {"workload": "serve-hybrid", "results": res},
+        "vs_baseline": None, "config": {"workload": f"serve-{kind}", "results": res},
     }))
 
 
 def main():
     args = parse_args()
-    if args.workload == "serve-hybrid":
-        return serve_hybrid(args)
+    if args.workload in ("serve-hybrid", "serve-moe"):
+        return serve_comparison(args, args.workload.split("-")[1])
     import colossalai_amd
     from colossalai_amd.models import LLAMA_CONFIGS, LlamaForCausalLM, llama_flops_per_token
 

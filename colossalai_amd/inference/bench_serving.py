@@ -1,7 +1,9 @@
-"""Serving throughput of the hybrid (paged window attention + recurrent state)
-model next to a Llama of equal width, depth and parameter budget, both through
-``ContinuousBatchEngine``: prefill tokens/s of one long prompt and decode
-tokens/s of a batch of running sequences. Random weights, synthetic tokens.
+"""Serving throughput of the ragged-step models next to a Llama of equal width,
+depth and per-token work, all through ``ContinuousBatchEngine``: prefill tokens/s
+of one long prompt and decode tokens/s of a batch of running sequences. Random
+weights, synthetic tokens. Two comparisons: the Kipirax hybrid (paged window
+attention + recurrent state) and Mubutar (sink-softmax attention with shared
+keys, routed experts).
 """
 
 import json
@@ -10,11 +12,12 @@ from typing import Dict, List
 
 import torch
 
-from ..models import KipiraxConfig, KipiraxForCausalLM, LlamaConfig, LlamaForCausalLM
+from ..models import (KipiraxConfig, KipiraxForCausalLM, LlamaConfig, LlamaForCausalLM, MubutarConfig,
+                      MubutarForCausalLM)
 from .config import InferenceConfig
 from .paged_engine import ContinuousBatchEngine
 
-__all__ = ["SIZES", "hybrid_config", "llama_config", "run_serving_comparison"]
+__all__ = ["SIZES", "hybrid_config", "llama_config", "moe_config", "run_serving_comparison"]
 
 # width, layers, heads, kv_heads, head size, vocab
 SIZES = {
@@ -37,9 +40,34 @@ def hybrid_config(s: dict, max_positions: int, window: int = 1024, keep_first: i
                          norm_groups=4, logit_softcap=30.0)
 
 
+def _inter(width: int) -> int:
+    return (8 * width // 3 + 255) // 256 * 256
+
+
+def moe_config(s: dict, experts: int = 32, top: int = 6) -> MubutarConfig:
+    """Even layers: own keys + dense gated feed-forward of Llama's size. Odd layers: the keys of
+    the layer before + routed experts whose active matrices (top experts + shared, two matrices
+    each) do the work of Llama's three."""
+    W, H, G, D = s["width"], s["heads"], s["kv_heads"], s["dim"]
+    inter = _inter(W)
+    ff = W // 2
+    shared = (3 * inter // 2 - top * ff + 127) // 128 * 128
+    att = dict(dim=D, heads=H, kv_heads=G, vdim=D, scale=D ** -0.5, softcap=50.0)
+    layers = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            layers.append(dict(type="attention", mixer=att, mlp=dict(kind="dense", ff=inter)))
+        else:
+            layers.append(dict(type="attention", mixer=dict(att, kv_from=i - 1),
+                               mlp=dict(kind="moe", expert=dict(ff=ff), shared=dict(ff=shared),
+                                        router=dict(experts=experts, top=top, groups=dict(count=8, keep=4)))))
+    return MubutarConfig(vocab=s["vocab"], width=W, layers=layers, norm_eps=1e-6, embedding_scale=W ** 0.5,
+                         logit_scale=1.0)
+
+
 def llama_config(s: dict, max_positions: int) -> LlamaConfig:
     # gate/up/down of 8/3 W carry the parameters of the hybrid's up/down of 4 W
-    inter = (8 * s["width"] // 3 + 255) // 256 * 256
+    inter = _inter(s["width"])
     return LlamaConfig(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=inter,
                        num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
                        num_key_value_heads=s["kv_heads"], max_position_embeddings=max_positions)
@@ -66,19 +94,33 @@ def _timed(fn, repeats: int) -> float:
 
 
 def _hybrid_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
-    page = 64
     cfg = hybrid_config(s, max_positions=max(prompt, context + steps + 8) + 8)
-    model = _random(KipiraxForCausalLM(cfg), torch.bfloat16)
+    return _ragged_numbers(_random(KipiraxForCausalLM(cfg), torch.bfloat16), cfg.vocab, prompt, batch, context, steps)
+
+
+def _moe_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
+    cfg = moe_config(s)
+    model = _random(MubutarForCausalLM(cfg), torch.bfloat16)
+    for layer in model.layers:  # the router stays float32
+        if hasattr(layer.mlp, "router"):
+            layer.mlp.router.data = layer.mlp.router.data.float()
+        layer.mix.in_proj.bias.data = layer.mix.in_proj.bias.data.to(torch.bfloat16)
+    out = _ragged_numbers(model, cfg.vocab, prompt, batch, context, steps)
+    return out
+
+
+def _ragged_numbers(model, vocab: int, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
+    page = 64
     blocks = max(prompt, batch * (context + steps + page)) // page + batch + 2
     eng = ContinuousBatchEngine(model, InferenceConfig(max_batch_size=batch + 1), num_blocks=blocks, block_size=page)
-    toks = torch.randint(0, cfg.vocab, (prompt,)).tolist()
+    toks = torch.randint(0, vocab, (prompt,)).tolist()
 
     def prefill():
         eng.run_ragged([("p", toks, [prompt - 1])])
         eng.close_sequence("p")
 
     t_prefill = _timed(prefill, 3)
-    ctx = torch.randint(0, cfg.vocab, (batch, context)).tolist()
+    ctx = torch.randint(0, vocab, (batch, context)).tolist()
     eng.run_ragged([(i, ctx[i], [context - 1]) for i in range(batch)])
 
     def decode():
@@ -121,11 +163,13 @@ def _llama_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -
 
 
 def run_serving_comparison(sizes: List[str], prompt: int = 4096, batch: int = 16, context: int = 1024,
-                           steps: int = 32) -> dict:
+                           steps: int = 32, kind: str = "hybrid") -> dict:
+    """``kind``: "hybrid" (Kipirax) or "moe" (Mubutar), each next to Llama."""
+    ours = {"hybrid": _hybrid_numbers, "moe": _moe_numbers}[kind]
     out = {}
     for name in sizes:
         s = SIZES[name]
-        out[name] = {"hybrid": _hybrid_numbers(s, prompt, batch, context, steps),
+        out[name] = {kind: ours(s, prompt, batch, context, steps),
                      "llama": _llama_numbers(s, prompt, batch, context, steps),
                      "shape": dict(s, prompt=prompt, batch=batch, context=context)}
     return out

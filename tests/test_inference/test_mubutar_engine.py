@@ -188,18 +188,44 @@ def test_greedy_generation_through_scheduler(device):
     assert eng.kv.free_blocks == 40 and eng.state.free_slots == 2
 
 
-def test_replay_writes_the_oracles_logits(tmp_path):
-    """bin/trace_run on a checkpoint folder on disk (bfloat16 tensors, as a
-    checkpoint holds them), float32 serving on the CPU."""
+def checkpoint_folder(tmp_path):
+    """A checkpoint folder on disk, bfloat16 tensors as a checkpoint holds them."""
     from safetensors.torch import save_file
 
     cfg = dict(CFG, vocab=30, layers=CFG["layers"][:2])
     W = {k: v.to(torch.bfloat16) for k, v in O.random_weights(cfg, seed=11).items()}
-    Wf = {k: v.float() for k, v in W.items()}
-    model_dir, out_dir = tmp_path / "model", tmp_path / "out"
+    model_dir = tmp_path / "model"
     model_dir.mkdir()
     (model_dir / "config.json").write_text(json.dumps(cfg))
     save_file({k: v.contiguous() for k, v in W.items()}, str(model_dir / "model.safetensors"))
+    return cfg, {k: v.float() for k, v in W.items()}, model_dir
+
+
+def test_command_line_lists_and_generates(tmp_path):
+    """`models` names the architecture; `generate` loads the folder through the
+    registry and decodes greedily through the engine's scheduler."""
+    cfg, Wf, model_dir = checkpoint_folder(tmp_path)
+    env = dict(os.environ, PYTHONPATH=ROOT, CUDA_VISIBLE_DEVICES="", HIP_VISIBLE_DEVICES="")
+    cli = [sys.executable, "-m", "colossalai_amd.cli.cli"]
+    r = subprocess.run(cli + ["models"], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0 and "mubutar" in r.stdout.split()
+    r = subprocess.run(cli + ["generate", "--model", str(model_dir), "--prompt-ids", "3,9,27,1,4;5,6", "--max-new-tokens", "4",
+                              "--dtype", "float32", "--max-step-tokens", "3"], capture_output=True, text=True, env=env,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [json.loads(l) for l in r.stdout.splitlines() if l.startswith("{")]
+    assert [l["prompt_ids"] for l in lines] == [[3, 9, 27, 1, 4], [5, 6]]
+    for l in lines:
+        seq = list(l["prompt_ids"])
+        for _ in range(4):
+            seq.append(int(O.forward(cfg, Wf, seq)[-1].argmax()))
+        assert l["output_ids"] == seq[len(l["prompt_ids"]):]
+
+
+def test_replay_writes_the_oracles_logits(tmp_path):
+    """bin/trace_run on a checkpoint folder on disk, float32 serving on the CPU."""
+    cfg, Wf, model_dir = checkpoint_folder(tmp_path)
+    out_dir = tmp_path / "out"
     a = torch.randint(0, 30, (21,), generator=torch.Generator().manual_seed(0)).tolist()
     b = torch.randint(0, 30, (9,), generator=torch.Generator().manual_seed(1)).tolist()
     steps = [
