@@ -135,16 +135,27 @@ void paged_kv_write(at::Tensor k, at::Tensor v, at::Tensor kpool, at::Tensor vpo
   HIP_CHECK_LAST();
 }
 
-// packed [N, 2F] = [gate | up], rows strided by ps -> out [N, F] = silu(gate) * up, formed in float32
-template <typename T>
+// packed [N, 2F] = [gate | up], rows strided by ps -> out [N, F] = silu(gate) * up, formed in float32.
+// VEC: eight elements per thread (F and the row stride are multiples of 8 and the base is aligned).
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ packed, long ps,
                                                        long N, int F) {
-  const long total = N * F;
+  constexpr int PER = VEC ? 8 : 1;
+  const long total = N * F / PER;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-    const long n = i / F;
-    const int f = (int)(i % F);
-    const float g = ldf(packed + n * ps + f), u = ldf(packed + n * ps + F + f);
-    stf(out + i, g * sigmoidf_(g) * u);
+    const long n = i * PER / F;
+    const int f = (int)(i * PER % F);
+    if (VEC) {
+      float g[8], u[8];
+      load8(packed + n * ps + f, g);
+      load8(packed + n * ps + F + f, u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = g[e] * sigmoidf_(g[e]) * u[e];
+      store8(out + n * F + f, g);
+    } else {
+      const float g = ldf(packed + n * ps + f), u = ldf(packed + n * ps + F + f);
+      stf(out + i, g * sigmoidf_(g) * u);
+    }
   }
 }
 
@@ -155,9 +166,14 @@ at::Tensor silu_mul(at::Tensor packed) {
   const int F = (int)(packed.size(1) / 2);
   at::Tensor out = at::empty({N, F}, packed.options());
   if (N * F == 0) return out;
+  const bool vec = F % 8 == 0 && packed.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(packed.data_ptr()) % 32 == 0;
   SERVING_DISPATCH_ACT(packed, T, {
-    hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(capped_grid((N * F + 255) / 256, 4096)), dim3(256), 0, stream(),
-                       ptr<T>(out), ptr<T>(packed), (long)packed.stride(0), N, F);
+    if (vec)
+      hipLaunchKernelGGL((silu_mul_kernel<T, true>), dim3(capped_grid((N * F / 8 + 255) / 256, 8192)), dim3(256), 0, stream(),
+                         ptr<T>(out), ptr<T>(packed), (long)packed.stride(0), N, F);
+    else
+      hipLaunchKernelGGL((silu_mul_kernel<T, false>), dim3(capped_grid((N * F + 255) / 256, 4096)), dim3(256), 0, stream(),
+                         ptr<T>(out), ptr<T>(packed), (long)packed.stride(0), N, F);
   });
   HIP_CHECK_LAST();
   return out;

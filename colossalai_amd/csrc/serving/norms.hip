@@ -26,12 +26,14 @@ __global__ __launch_bounds__(256) void grouped_rms_norm_kernel(
   const int g = (int)(unit % groups);
   const long base = (row * groups + g) * (long)gs;
   float ssq = 0.0f;
-  for (int i = lane; i < gs; i += 64) {
+#pragma unroll 8
+  for (int i = lane; i < gs; i += 64) {  // unrolled: the loads of a row are in flight together
     const float v = ldf(x + base + i);
     ssq += v * v;
   }
   ssq = wave_reduce_sum(ssq);
   const float inv = 1.0f / sqrtf(ssq / (float)gs + eps);
+#pragma unroll 8
   for (int i = lane; i < gs; i += 64) {
     const float y = ldf(x + base + i) * inv * w[g * gs + i];
     if (residual != nullptr) residual[base + i] += y;
@@ -205,6 +207,7 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(
   const long row = blockIdx.x;
   float* rr = residual + row * W;
   float ssq = 0.0f;
+#pragma unroll 4
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float add = ldf(a + row * W + i);
     if (b != nullptr) add += ldf(b + row * W + i);

@@ -246,7 +246,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int hl = blockIdx.z * (nthreads >> 6) + wid;  // head inside the group
   const bool head_ok = hl < rep;
   const int h = g * rep + (head_ok ? hl : 0);
-  int tile = blockIdx.x, b = 0;
+  // Under a causal mask a late tile of a long prompt has many more key tiles than an early one. Rows of the grid
+  // (kv head, pass) walk the tiles alternately from the back and from the front, switching with every 256 blocks of
+  // dispatch order, so that blocks which come to share a CU tend to pair a long tile with a short one and the
+  // longest tiles start first.
+  const bool from_back = ((gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) >> 8 & 1) == 0;
+  int tile = from_back ? gridDim.x - 1 - blockIdx.x : blockIdx.x, b = 0;
   for (;; ++b) {  // the grid holds exactly sum_b ceil(count_b / 32) tiles
     const int nt = (cu[b + 1] - cu[b] + 31) >> 5;
     if (tile < nt) break;
@@ -276,7 +281,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int sink_tiles = (n_sink + 31) >> 5;
   const int tiles_n = sink_tiles + ((p1 - wstart) >> 5) + 1;
 
-  // staging: chunk c of a tile = key c / (row chunks), 8 elements starting at 8 * (c % row chunks)
+  // staging: key chunk c = key c / (row chunks), 8 elements starting at 8 * (c % row chunks), stored as a row;
+  // value chunk c = key c % 32, 8 channels starting at 8 * (c / 32): the values are stored transposed, two bytes at
+  // a time, and with neighbouring threads on neighbouring keys these stores spread over the LDS banks
   constexpr int KR = (KCH + 255) / 256, VR = (VCH + 255) / 256;  // chunks per thread of the 256
   bf16x8_v rk[KR], rv[VR];
   auto tile_base = [&](int it) { return it < sink_tiles ? it * 32 : wstart + (it - sink_tiles) * 32; };
@@ -298,8 +305,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     for (int r = 0; r < VR; ++r) {
       const int c = tid + nthreads * r;
       if (c < VCH) {
-        const int off = 8 * (c % (Dv / 8));
-        rv[r] = off < Dvr ? ld_g16b(vpool + (pool_row(kbase + c / (Dv / 8)) * G + g) * Dvr + off) : zero8;
+        const int off = 8 * (c >> 5);
+        rv[r] = off < Dvr ? ld_g16b(vpool + (pool_row(kbase + (c & 31)) * G + g) * Dvr + off) : zero8;
       }
     }
   };
@@ -315,7 +322,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     for (int r = 0; r < VR; ++r) {
       const int c = tid + nthreads * r;
       if (c < VCH) {
-        const int kk = c / (Dv / 8), dv0 = 8 * (c % (Dv / 8));
+        const int kk = c & 31, dv0 = 8 * (c >> 5);
         // contraction slot of key kk: the order in which the C layout of S^T hands the weights to P^T
         const int r16 = kk & 15;
         const int slot = (kk & 16) + ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);

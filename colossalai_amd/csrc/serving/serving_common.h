@@ -34,6 +34,16 @@ DEV_INLINE void load8(const bf16s* p, float* o) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = bf2f((bf16s)a[e]);
 }
+DEV_INLINE void store8(float* p, const float* v) {
+  *reinterpret_cast<float4v*>(p) = float4v{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<float4v*>(p + 4) = float4v{v[4], v[5], v[6], v[7]};
+}
+DEV_INLINE void store8(bf16s* p, const float* v) {
+  short8 a;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) a[e] = (short)f2bf(v[e]);
+  *reinterpret_cast<short8*>(p) = a;
+}
 // two consecutive elements
 DEV_INLINE void load2(const float* p, float& a, float& b) {
   const float2v t = *reinterpret_cast<const float2v*>(p);
