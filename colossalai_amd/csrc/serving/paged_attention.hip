@@ -291,14 +291,29 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const int jc = min(j, p1);  // keys past the sequence's end are masked; read a row that exists
     return ((long)bt[jc >> page_shift] << page_shift) + (jc & page_mask);
   };
-  auto fetch = [&](int it) {
+  // The page-table lookups of a tile run one tile ahead of its key/value loads (two ahead of its use), so that a
+  // load's address never waits for a lookup issued in the same iteration.
+  int krow[KR], vrow[VR];
+  auto lookup = [&](int it) {
     const int kbase = tile_base(it);
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+      const int c = tid + nthreads * r;
+      krow[r] = c < KCH ? (int)pool_row(kbase + c / (D / 8)) : 0;
+    }
+#pragma unroll
+    for (int r = 0; r < VR; ++r) {
+      const int c = tid + nthreads * r;
+      vrow[r] = c < VCH ? (int)pool_row(kbase + (c & 31)) : 0;
+    }
+  };
+  auto fetch = [&]() {  // the tile whose rows the last lookup left in krow / vrow
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
       const int c = tid + nthreads * r;
       if (c < KCH) {
         const int off = 8 * (c % (D / 8));
-        rk[r] = off < Dr ? ld_g16b(kpool + (pool_row(kbase + c / (D / 8)) * G + g) * Dr + off) : zero8;
+        rk[r] = off < Dr ? ld_g16b(kpool + ((long)krow[r] * G + g) * Dr + off) : zero8;
       }
     }
 #pragma unroll
@@ -306,7 +321,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       const int c = tid + nthreads * r;
       if (c < VCH) {
         const int off = 8 * (c >> 5);
-        rv[r] = off < Dvr ? ld_g16b(vpool + (pool_row(kbase + (c & 31)) * G + g) * Dvr + off) : zero8;
+        rv[r] = off < Dvr ? ld_g16b(vpool + ((long)vrow[r] * G + g) * Dvr + off) : zero8;
       }
     }
   };
@@ -355,13 +370,18 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < 16; ++i) row_bias[i] = sl2 * (float)((i & 3) + 8 * (i >> 2) + 4 * hf);
 
-  fetch(0);
+  lookup(0);
+  fetch();
+  if (tiles_n > 1) lookup(1);
   stash(0);
   __syncthreads();
   for (int it = 0; it < tiles_n; ++it) {
     const int buf = it & 1;
     const bool more = it + 1 < tiles_n;
-    if (more) fetch(it + 1);
+    if (more) {
+      fetch();
+      if (it + 2 < tiles_n) lookup(it + 2);
+    }
     if (head_ok) {
       const bool sink = it < sink_tiles;
       const int kbase = tile_base(it);
