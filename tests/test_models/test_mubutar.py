@@ -224,6 +224,14 @@ SHAPES = {
                                 dict(type="attention", mixer=dict(dim=8, heads=4, kv_heads=1, vdim=24, scale=0.2, softcap=1.5,
                                                                   kv_from=1),
                                      mlp=dict(kind="dense", ff=24))]),
+    # nothing a multiple of 8 or of the wave: scalar loads everywhere, three query heads on one kv head
+    "odd-sizes": dict(vocab=37, width=36, embedding=dict(scale=1.7), logit_scale=0.9, norm=dict(eps=1e-6),
+                      layers=[dict(type="attention", mixer=dict(dim=6, heads=3, kv_heads=1, vdim=5, scale=0.41, softcap=11.0),
+                                   mlp=dict(kind="moe", expert=dict(ff=10), shared=dict(ff=7),
+                                            router=dict(experts=9, top=4, groups=dict(count=3, keep=2)))),
+                              dict(type="attention", mixer=dict(dim=6, heads=3, kv_heads=1, vdim=5, scale=0.41, softcap=11.0,
+                                                                kv_from=0),
+                                   mlp=dict(kind="dense", ff=21))]),
 }
 
 
