@@ -1,4 +1,6 @@
-// pybind bindings for colossalai_amd._C_serving (ragged serving kernels, gfx950).
+// pybind bindings for colossalai_amd._C_serving (ragged serving kernels every ragged model uses:
+// paged attention, norms, element-wise steps, router and experts; gfx950). The kernels of
+// fixed-size sequence state live in colossalai_amd._C_serving_state.
 #include <torch/extension.h>
 
 namespace cai {
@@ -15,13 +17,6 @@ at::Tensor head_rms_norm_gate(at::Tensor x, at::Tensor weight, double eps, c10::
                               at::ScalarType out_dtype);
 at::Tensor merge_rms_norm(at::Tensor a, at::Tensor wa, at::Tensor b, at::Tensor wb, double eps, at::Tensor out_w,
                           int64_t groups, at::Tensor residual);
-at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> tail, at::Tensor cu, at::Tensor start,
-                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype);
-at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta_logit, at::Tensor dt,
-                            at::Tensor A_log, at::Tensor dt_bias, at::Tensor state, at::Tensor cu, at::Tensor start,
-                            at::Tensor slots, double unit_eps, double q_scale);
-at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, at::Tensor f_bias, at::Tensor lower,
-                                at::Tensor state, at::Tensor cu, at::Tensor start, at::Tensor slots);
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
@@ -47,9 +42,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("grouped_rms_norm", &s::grouped_rms_norm, "grouped RMS norm, optional in-place residual add");
   m.def("head_rms_norm_gate", &s::head_rms_norm_gate, "per-head RMS norm with shared weight and sigmoid gate");
   m.def("merge_rms_norm", &s::merge_rms_norm, "average of two RMS-normed branches, group norm, residual add");
-  m.def("short_conv", &s::short_conv, "short causal depthwise convolution with carried tail");
-  m.def("gated_delta_rule", &s::gated_delta_rule, "gated delta rule with per-channel decay, carried state");
-  m.def("tied_gate_recurrence", &s::tied_gate_recurrence, "HGRN2-style recurrence, carried state");
   m.def("paged_attention", &s::paged_attention, "ragged paged attention: window, kept prefix, distance bias, gate, soft cap, sink");
   m.def("silu_mul", &s::silu_mul, "silu(gate) * up of a packed [N, 2F] tensor");
   m.def("add_rms_norm", &s::add_rms_norm, "residual += a (+ b) in place, then the RMS norm of the sum");

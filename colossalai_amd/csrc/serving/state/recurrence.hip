@@ -15,7 +15,7 @@
 // A prologue kernel turns the raw projections into float32 operands once per
 // token (unit-length q/k, decay from its logits, gates), so the sequential
 // loop holds no transcendental.
-#include "serving_common.h"
+#include "../serving_common.h"
 
 namespace cai {
 namespace serving {

@@ -5,7 +5,7 @@
 // the tail refresh (one thread owns all K-1 entries of a (sequence, channel),
 // reads them before it writes), so no element is read and written by
 // different threads of one launch.
-#include "serving_common.h"
+#include "../serving_common.h"
 
 namespace cai {
 namespace serving {

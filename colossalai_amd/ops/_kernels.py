@@ -46,45 +46,56 @@ def use_hip(*tensors: torch.Tensor) -> bool:
 
 
 # ---------------------------------------------------------------------------
-# colossalai_amd._C_serving: the ragged serving kernels (paged attention with
-# window / sinks / distance bias, matrix-state recurrences, short convolution,
-# token shift, grouped norms). It is a separate, small extension so that a
-# fresh checkout that only serves a model compiles these few files and not the
-# training kernels.
-_SERVING = None
+# The ragged serving kernels are two small extensions of their own, so that a
+# fresh checkout that only serves a model compiles the few files that model
+# needs and not the training kernels:
+#   colossalai_amd._C_serving        paged attention (window / sinks / distance bias / soft cap),
+#                                    norms, element-wise steps, token shift, router and experts;
+#   colossalai_amd._C_serving_state  fixed-size per-sequence state: matrix-state recurrences and
+#                                    the short convolution (only models with such layers load it).
+_LOADED = {}
 
 
-def build_serving_extension() -> None:
-    """Compile colossalai_amd._C_serving in-tree (gfx950) with the repo's setup.py."""
+def build_serving_extension(which: str = "serving") -> None:
+    """Compile one serving extension in-tree (gfx950) with the repo's setup.py."""
     import os
     import subprocess
     import sys
 
     root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-    env = dict(os.environ, PYTORCH_ROCM_ARCH="gfx950", COLOSSALAI_AMD_EXTENSIONS="serving")
+    env = dict(os.environ, PYTORCH_ROCM_ARCH="gfx950", COLOSSALAI_AMD_EXTENSIONS=which)
     subprocess.run([sys.executable, "setup.py", "build_ext", "--inplace"], cwd=root, env=env, check=True,
                    stdout=sys.stderr)
 
 
-def serving_kernels(build_if_missing: bool = True):
-    """Return colossalai_amd._C_serving, compiling it once if it is not built."""
-    global _SERVING
-    if _SERVING is None:
+def _load(which: str, build_if_missing: bool):
+    if which not in _LOADED:
         import importlib
 
+        name = "colossalai_amd._C_" + which
         try:
-            _SERVING = importlib.import_module("colossalai_amd._C_serving")
+            _LOADED[which] = importlib.import_module(name)
         except ImportError:
             if not build_if_missing:
                 raise
-            build_serving_extension()
+            build_serving_extension(which)
             importlib.invalidate_caches()
-            _SERVING = importlib.import_module("colossalai_amd._C_serving")
-    return _SERVING
+            _LOADED[which] = importlib.import_module(name)
+    return _LOADED[which]
+
+
+def serving_kernels(build_if_missing: bool = True):
+    """Return colossalai_amd._C_serving, compiling it once if it is not built."""
+    return _load("serving", build_if_missing)
+
+
+def serving_state_kernels(build_if_missing: bool = True):
+    """Return colossalai_amd._C_serving_state, compiling it once if it is not built."""
+    return _load("serving_state", build_if_missing)
 
 
 def use_serving_hip(*tensors: torch.Tensor) -> bool:
     """True when the serving ops must take their HIP path (tensors on the GPU);
-    ``serving_kernels()`` then loads, or compiles, the extension — there is no
-    eager fallback on a GPU."""
+    ``serving_kernels()`` / ``serving_state_kernels()`` then load, or compile,
+    the extension — there is no eager fallback on a GPU."""
     return all(t.is_cuda for t in tensors if isinstance(t, torch.Tensor))

@@ -20,7 +20,7 @@ state are float32 whatever the activation dtype is.
 import torch
 import torch.nn.functional as F
 
-from ._kernels import serving_kernels, use_serving_hip as use_hip
+from ._kernels import serving_state_kernels as serving_kernels, use_serving_hip as use_hip
 from .ragged import RaggedBatch
 
 __all__ = ["gated_delta_rule", "gated_delta_rule_ref", "tied_gate_recurrence", "tied_gate_recurrence_ref"]

@@ -9,7 +9,7 @@ mid-sequence sees the inputs of earlier steps.
 import torch
 import torch.nn.functional as F
 
-from ._kernels import serving_kernels, use_serving_hip as use_hip
+from ._kernels import serving_state_kernels as serving_kernels, use_serving_hip as use_hip
 from .ragged import RaggedBatch
 
 __all__ = ["short_conv", "short_conv_ref"]

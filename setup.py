@@ -23,6 +23,9 @@ cpu_sources = [os.path.join(CSRC_CPU, f) for f in sorted(os.listdir(CSRC_CPU)) i
 SERVING = os.path.join(CSRC, "serving")
 serving_sources = [os.path.join(SERVING, f) for f in sorted(os.listdir(SERVING))
                    if f.endswith((".hip", ".cpp")) and not f.endswith("_hip.hip")]
+STATE = os.path.join(SERVING, "state")
+state_sources = [os.path.join(STATE, f) for f in sorted(os.listdir(STATE))
+                 if f.endswith((".hip", ".cpp")) and not f.endswith("_hip.hip")]
 # -packed-fp32-ops off: the compiler then emits no packed float32 arithmetic
 NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -51,6 +54,16 @@ serving_ext = CUDAExtension(
     },
 )
 
+# kernels of fixed-size per-sequence state (recurrences, short convolution): only models with such layers need them
+state_ext = CUDAExtension(
+    name="colossalai_amd._C_serving_state",
+    sources=state_sources,
+    extra_compile_args={
+        "cxx": ["-O3", "-std=c++17"],
+        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"] + NO_PACKED_FP32,
+    },
+)
+
 cpu_ext = CppExtension(
     name="colossalai_amd._C_cpu",
     sources=cpu_sources,
@@ -62,8 +75,8 @@ setup(
     name="colossalai_amd",
     version="0.1.0",
     packages=find_packages(include=["colossalai_amd", "colossalai_amd.*"]),
-    # COLOSSALAI_AMD_EXTENSIONS=serving builds just the serving kernels
-    ext_modules=[serving_ext] if os.environ.get("COLOSSALAI_AMD_EXTENSIONS") == "serving"
-    else [ext, cpu_ext, serving_ext],
+    # COLOSSALAI_AMD_EXTENSIONS=serving / serving_state builds just that one serving extension
+    ext_modules={"serving": [serving_ext], "serving_state": [state_ext]}.get(
+        os.environ.get("COLOSSALAI_AMD_EXTENSIONS"), [ext, cpu_ext, serving_ext, state_ext]),
     cmdclass={"build_ext": BuildExtension.with_options(use_ninja=True)},
 )
