@@ -253,19 +253,43 @@ at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at:
 }
 
 // ------------------------------------------------------------------ combine
-// out[n, w] = base[n, w] + sum_j weights[n, j] * y[inv[n, j], w], slots in order, float32
-template <typename T, typename TB>
+// out[n, w] = base[n, w] + sum_j weights[n, j] * y[inv[n, j], w], slots in order, float32.
+// VEC: eight columns per thread (W a multiple of 8, 32-byte aligned operands).
+template <typename T, typename TB, bool VEC>
 __global__ __launch_bounds__(256) void expert_combine_kernel(
     float* __restrict__ out, const T* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
     const TB* __restrict__ base, int top, int W, long rows) {
   const long n = blockIdx.x;
-  for (int w = threadIdx.x; w < W; w += blockDim.x) {
-    float acc = base != nullptr ? ldf(base + n * W + w) : 0.0f;
-    for (int j = 0; j < top; ++j) {
-      const long r = inv[n * top + j];
-      if (r >= 0 && r < rows) acc += weights[n * top + j] * ldf(y + r * W + w);
+  if (VEC) {
+    for (int w = threadIdx.x * 8; w < W; w += blockDim.x * 8) {
+      float acc[8];
+      if (base != nullptr) {
+        load8(base + n * W + w, acc);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+      }
+      for (int j = 0; j < top; ++j) {
+        const long r = inv[n * top + j];
+        if (r >= 0 && r < rows) {
+          float v[8];
+          load8(y + r * W + w, v);
+          const float wj = weights[n * top + j];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] += wj * v[e];
+        }
+      }
+      store8(out + n * W + w, acc);
     }
-    out[n * W + w] = acc;
+  } else {
+    for (int w = threadIdx.x; w < W; w += blockDim.x) {
+      float acc = base != nullptr ? ldf(base + n * W + w) : 0.0f;
+      for (int j = 0; j < top; ++j) {
+        const long r = inv[n * top + j];
+        if (r >= 0 && r < rows) acc += weights[n * top + j] * ldf(y + r * W + w);
+      }
+      out[n * W + w] = acc;
+    }
   }
 }
 
@@ -283,18 +307,28 @@ at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10:
   }
   at::Tensor out = at::empty({N, W}, y.options().dtype(at::kFloat));
   if (N == 0) return out;
+  auto al32 = [](const at::Tensor& t) { return reinterpret_cast<uintptr_t>(t.data_ptr()) % 32 == 0; };
+  const bool vec = W % 8 == 0 && al32(y) && al32(out) && (!base.has_value() || al32(*base));
+  const float* nobase = nullptr;
+#define COMBINE_LAUNCH(TB_, bp)                                                                                       \
+  do {                                                                                                                \
+    if (vec)                                                                                                          \
+      hipLaunchKernelGGL((expert_combine_kernel<T, TB_, true>), dim3((unsigned)N), dim3(256), 0, stream(),           \
+                         out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, top, W, \
+                         (long)y.size(0));                                                                            \
+    else                                                                                                              \
+      hipLaunchKernelGGL((expert_combine_kernel<T, TB_, false>), dim3((unsigned)N), dim3(256), 0, stream(),          \
+                         out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, top, W, \
+                         (long)y.size(0));                                                                            \
+  } while (0)
   SERVING_DISPATCH_ACT(y, T, {
     if (base.has_value()) {
-      SERVING_DISPATCH_ACT(*base, TB, {
-        hipLaunchKernelGGL((expert_combine_kernel<T, TB>), dim3((unsigned)N), dim3(256), 0, stream(), out.data_ptr<float>(),
-                           ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), ptr<TB>(*base), top, W, (long)y.size(0));
-      });
+      SERVING_DISPATCH_ACT(*base, TB, { COMBINE_LAUNCH(TB, ptr<TB>(*base)); });
     } else {
-      hipLaunchKernelGGL((expert_combine_kernel<T, float>), dim3((unsigned)N), dim3(256), 0, stream(), out.data_ptr<float>(),
-                         ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), (const float*)nullptr, top, W,
-                         (long)y.size(0));
+      COMBINE_LAUNCH(float, nobase);
     }
   });
+#undef COMBINE_LAUNCH
   HIP_CHECK_LAST();
   return out;
 }

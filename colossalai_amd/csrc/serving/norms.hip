@@ -221,6 +221,50 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(
   for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + row * W + i, rr[i] * inv * w[i]);
 }
 
+// Row-in-registers form for rows of up to 2048 * CH elements (W a multiple of 8, 32-byte aligned
+// operands): each thread owns CH chunks of 8 consecutive elements, reads every operand once with
+// 16/32-byte loads, keeps the summed row in registers across the reduction and writes residual and
+// normed row once.
+template <typename TA, typename TB, typename TO, int CH>
+__global__ __launch_bounds__(256) void add_rms_norm_rows_kernel(
+    TO* __restrict__ out, float* __restrict__ residual, const TA* __restrict__ a, const TB* __restrict__ b,
+    const float* __restrict__ w, int W, float eps) {
+  __shared__ float red[8];
+  const long row = blockIdx.x;
+  float r[CH][8];
+  float ssq = 0.0f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (threadIdx.x + 256 * c) * 8;
+    if (i < W) {
+      float av[8], bv[8];
+      load8(residual + row * W + i, r[c]);
+      load8(a + row * W + i, av);
+      if (b != nullptr) load8(b + row * W + i, bv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        r[c][e] += b != nullptr ? av[e] + bv[e] : av[e];
+        ssq += r[c][e] * r[c][e];
+      }
+      store8(residual + row * W + i, r[c]);
+    }
+  }
+  if (w == nullptr) return;
+  ssq = block_reduce_sum(ssq, red);
+  const float inv = 1.0f / sqrtf(ssq / (float)W + eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (threadIdx.x + 256 * c) * 8;
+    if (i < W) {
+      float wv[8];
+      load8(w + i, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wv[e] *= r[c][e] * inv;
+      store8(out + row * W + i, wv);
+    }
+  }
+}
+
 c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::optional<at::Tensor> b,
                                        c10::optional<at::Tensor> weight, double eps, at::ScalarType out_dtype) {
   check_act(a, "a");
@@ -245,20 +289,36 @@ c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::o
   if (N > 0) {
     // without a weight nothing is written through `out`: any instantiation of TO will do
     const at::Tensor& like = weight.has_value() ? out : residual;
+    auto al32 = [](const at::Tensor& t) { return reinterpret_cast<uintptr_t>(t.data_ptr()) % 32 == 0; };
+    const bool rows = W % 8 == 0 && W <= 2048 * 4 && al32(residual) && al32(a) && (!b.has_value() || al32(*b)) &&
+                      (!weight.has_value() || (al32(out) && al32(w)));
+    const float* nob = nullptr;
+#define ADD_NORM_LAUNCH(TB_, bp)                                                                                        \
+  do {                                                                                                                  \
+    if (rows && W <= 2048)                                                                                              \
+      hipLaunchKernelGGL((add_rms_norm_rows_kernel<TA, TB_, TO, 1>), dim3((unsigned)N), dim3(256), 0, stream(), op,    \
+                         residual.data_ptr<float>(), ptr<TA>(a), bp, wp, W, (float)eps);                                \
+    else if (rows && W <= 4096)                                                                                         \
+      hipLaunchKernelGGL((add_rms_norm_rows_kernel<TA, TB_, TO, 2>), dim3((unsigned)N), dim3(256), 0, stream(), op,    \
+                         residual.data_ptr<float>(), ptr<TA>(a), bp, wp, W, (float)eps);                                \
+    else if (rows)                                                                                                      \
+      hipLaunchKernelGGL((add_rms_norm_rows_kernel<TA, TB_, TO, 4>), dim3((unsigned)N), dim3(256), 0, stream(), op,    \
+                         residual.data_ptr<float>(), ptr<TA>(a), bp, wp, W, (float)eps);                                \
+    else                                                                                                                \
+      hipLaunchKernelGGL((add_rms_norm_kernel<TA, TB_, TO>), dim3((unsigned)N), dim3(256), 0, stream(), op,            \
+                         residual.data_ptr<float>(), ptr<TA>(a), bp, wp, W, (float)eps);                                \
+  } while (0)
     SERVING_DISPATCH_ACT(a, TA, {
       SERVING_DISPATCH_ACT(like, TO, {
         TO* op = weight.has_value() ? ptr<TO>(out) : (TO*)nullptr;
         if (b.has_value()) {
-          SERVING_DISPATCH_ACT(*b, TB, {
-            hipLaunchKernelGGL((add_rms_norm_kernel<TA, TB, TO>), dim3((unsigned)N), dim3(256), 0, stream(), op,
-                               residual.data_ptr<float>(), ptr<TA>(a), ptr<TB>(*b), wp, W, (float)eps);
-          });
+          SERVING_DISPATCH_ACT(*b, TB, { ADD_NORM_LAUNCH(TB, ptr<TB>(*b)); });
         } else {
-          hipLaunchKernelGGL((add_rms_norm_kernel<TA, float, TO>), dim3((unsigned)N), dim3(256), 0, stream(), op,
-                             residual.data_ptr<float>(), ptr<TA>(a), (const float*)nullptr, wp, W, (float)eps);
+          ADD_NORM_LAUNCH(float, nob);
         }
       });
     });
+#undef ADD_NORM_LAUNCH
     HIP_CHECK_LAST();
   }
   if (!weight.has_value()) return c10::nullopt;

@@ -262,7 +262,7 @@ def test_sink_with_tiny_scores_halves_nothing_by_accident():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W", [96, 1000])
+@pytest.mark.parametrize("W", [96, 1000, 2600, 5000, 100, 9000])  # rows held in registers (1, 2, 4 chunks), re-read rows
 def test_add_rms_norm(dtype, W):
     torch.manual_seed(10)
     x, w = torch.randn(19, W) * 4, torch.randn(W)
