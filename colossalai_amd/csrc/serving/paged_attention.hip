@@ -19,6 +19,7 @@ namespace serving {
 
 constexpr int ATT_WAVES = 16;  // most waves of a block: they split the key blocks of one (token, kv head)
 constexpr int RC_MAX = 4;      // most query heads of a kv head's group that one block handles together
+constexpr int MFMA_TILES_PER_STEP = 2;  // 32-key tiles the matrix-core kernel stages and multiplies between two barriers
 
 template <int CTRL>
 DEV_INLINE float dpp_add(float v) {
@@ -238,7 +239,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   constexpr int VP = 40;               // transposed value row pitch: 32 key slots + 8
   constexpr int KT = 32 * KP, VTT = Dv * VP;   // elements of one staged tile
   constexpr int KCH = 32 * D / 8, VCH = 32 * Dv / 8;  // 16-byte chunks of a key / value tile
-  extern __shared__ __align__(16) bf16s tiles[];  // [2][KT + VTT]
+  constexpr int TP = MFMA_TILES_PER_STEP;
+  extern __shared__ __align__(16) bf16s tiles[];  // [2][TP][KT + VTT]
   constexpr int nthreads = 256;  // always four waves: those beyond the group's heads only help staging
   const int tid = threadIdx.x;
   const int wid = tid >> 6, lane = tid & 63;
@@ -285,7 +287,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   // value chunk c = key c % 32, 8 channels starting at 8 * (c / 32): the values are stored transposed, two bytes at
   // a time, and with neighbouring threads on neighbouring keys these stores spread over the LDS banks
   constexpr int KR = (KCH + 255) / 256, VR = (VCH + 255) / 256;  // chunks per thread of the 256
-  bf16x8_v rk[KR], rv[VR];
+  // TP key tiles are staged, and multiplied, between two barriers: their loads are all in flight over the
+  // products of the TP tiles before them
+  bf16x8_v rk[TP][KR], rv[TP][VR];
   auto tile_base = [&](int it) { return it < sink_tiles ? it * 32 : wstart + (it - sink_tiles) * 32; };
   auto pool_row = [&](int j) {
     const int jc = min(j, p1);  // keys past the sequence's end are masked; read a row that exists
@@ -293,58 +297,67 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   };
   // The page-table lookups of a tile run one tile ahead of its key/value loads (two ahead of its use), so that a
   // load's address never waits for a lookup issued in the same iteration.
-  int krow[KR], vrow[VR];
-  auto lookup = [&](int it) {
-    const int kbase = tile_base(it);
+  int krow[TP][KR], vrow[TP][VR];
+  auto lookup = [&](int step) {
 #pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      const int c = tid + nthreads * r;
-      krow[r] = c < KCH ? (int)pool_row(kbase + c / (D / 8)) : 0;
-    }
+    for (int u = 0; u < TP; ++u) {
+      const int kbase = tile_base(step * TP + u);  // a tile past the last one reads rows that exist and is not used
 #pragma unroll
-    for (int r = 0; r < VR; ++r) {
-      const int c = tid + nthreads * r;
-      vrow[r] = c < VCH ? (int)pool_row(kbase + (c & 31)) : 0;
-    }
-  };
-  auto fetch = [&]() {  // the tile whose rows the last lookup left in krow / vrow
+      for (int r = 0; r < KR; ++r) {
+        const int c = tid + nthreads * r;
+        krow[u][r] = c < KCH ? (int)pool_row(kbase + c / (D / 8)) : 0;
+      }
 #pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      const int c = tid + nthreads * r;
-      if (c < KCH) {
-        const int off = 8 * (c % (D / 8));
-        rk[r] = off < Dr ? ld_g16b(kpool + ((long)krow[r] * G + g) * Dr + off) : zero8;
+      for (int r = 0; r < VR; ++r) {
+        const int c = tid + nthreads * r;
+        vrow[u][r] = c < VCH ? (int)pool_row(kbase + (c & 31)) : 0;
       }
     }
+  };
+  auto fetch = [&]() {  // the tiles whose rows the last lookup left in krow / vrow
 #pragma unroll
-    for (int r = 0; r < VR; ++r) {
-      const int c = tid + nthreads * r;
-      if (c < VCH) {
-        const int off = 8 * (c >> 5);
-        rv[r] = off < Dvr ? ld_g16b(vpool + ((long)vrow[r] * G + g) * Dvr + off) : zero8;
+    for (int u = 0; u < TP; ++u) {
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        const int c = tid + nthreads * r;
+        if (c < KCH) {
+          const int off = 8 * (c % (D / 8));
+          rk[u][r] = off < Dr ? ld_g16b(kpool + ((long)krow[u][r] * G + g) * Dr + off) : zero8;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < VR; ++r) {
+        const int c = tid + nthreads * r;
+        if (c < VCH) {
+          const int off = 8 * (c >> 5);
+          rv[u][r] = off < Dvr ? ld_g16b(vpool + ((long)vrow[u][r] * G + g) * Dvr + off) : zero8;
+        }
       }
     }
   };
   auto stash = [&](int buf) {
-    bf16s* ks = tiles + buf * (KT + VTT);
-    bf16s* vt = ks + KT;
 #pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      const int c = tid + nthreads * r;
-      if (c < KCH) *reinterpret_cast<bf16x8_v*>(ks + (c / (D / 8)) * KP + 8 * (c % (D / 8))) = rk[r];
-    }
+    for (int u = 0; u < TP; ++u) {
+      bf16s* ks = tiles + (buf * TP + u) * (KT + VTT);
+      bf16s* vt = ks + KT;
 #pragma unroll
-    for (int r = 0; r < VR; ++r) {
-      const int c = tid + nthreads * r;
-      if (c < VCH) {
-        const int kk = c & 31, dv0 = 8 * (c >> 5);
-        // contraction slot of key kk: the order in which the C layout of S^T hands the weights to P^T
-        const int r16 = kk & 15;
-        const int slot = (kk & 16) + ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);
+      for (int r = 0; r < KR; ++r) {
+        const int c = tid + nthreads * r;
+        if (c < KCH) *reinterpret_cast<bf16x8_v*>(ks + (c / (D / 8)) * KP + 8 * (c % (D / 8))) = rk[u][r];
+      }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const __bf16 x = rv[r][e];
-          vt[(dv0 + e) * VP + slot] = *reinterpret_cast<const bf16s*>(&x);
+      for (int r = 0; r < VR; ++r) {
+        const int c = tid + nthreads * r;
+        if (c < VCH) {
+          const int kk = c & 31, dv0 = 8 * (c >> 5);
+          // contraction slot of key kk: the order in which the C layout of S^T hands the weights to P^T
+          const int r16 = kk & 15;
+          const int slot = (kk & 16) + ((r16 >> 2) & 1) * 8 + (r16 >> 3) * 4 + (r16 & 3);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const __bf16 x = rv[u][r][e];
+            vt[(dv0 + e) * VP + slot] = *reinterpret_cast<const bf16s*>(&x);
+          }
         }
       }
     }
@@ -370,23 +383,27 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < 16; ++i) row_bias[i] = sl2 * (float)((i & 3) + 8 * (i >> 2) + 4 * hf);
 
+  const int steps_n = (tiles_n + TP - 1) / TP;
   lookup(0);
   fetch();
-  if (tiles_n > 1) lookup(1);
+  if (steps_n > 1) lookup(1);
   stash(0);
   __syncthreads();
-  for (int it = 0; it < tiles_n; ++it) {
-    const int buf = it & 1;
-    const bool more = it + 1 < tiles_n;
+  for (int step = 0; step < steps_n; ++step) {
+    const int buf = step & 1;
+    const bool more = step + 1 < steps_n;
     if (more) {
       fetch();
-      if (it + 2 < tiles_n) lookup(it + 2);
+      if (step + 2 < steps_n) lookup(step + 2);
     }
-    if (head_ok) {
+#pragma unroll
+    for (int u = 0; u < TP; ++u) {
+      const int it = step * TP + u;
+      if (!head_ok || it >= tiles_n) continue;
       const bool sink = it < sink_tiles;
       const int kbase = tile_base(it);
       const int klimit = sink ? n_sink : p1 + 1;  // keys of this tile at or above it are not this tile's to count
-      const bf16s* ks = tiles + buf * (KT + VTT);
+      const bf16s* ks = tiles + (buf * TP + u) * (KT + VTT);
       const bf16s* vt = ks + KT;
       f32x16 sacc;
 #pragma unroll
@@ -515,14 +532,18 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
     const int rep = H / G, nw = 4;
     const dim3 grid((unsigned)num_tiles, (unsigned)G, (unsigned)((rep + nw - 1) / nw));
     const int ds = D <= 32 ? 2 : D <= 48 ? 3 : D <= 64 ? 4 : D <= 96 ? 6 : 8, vt = (Dv + 31) / 32;
-    const size_t msmem = (size_t)2 * (32 * (ds * 16 + 8) + vt * 32 * 40) * sizeof(bf16s);
-#define MFMA_CASE(DS_, VT_)                                                                                          \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<DS_, VT_>), grid, dim3(64 * nw), msmem, stream(), ptr<bf16s>(out), \
-                     ptr<bf16s>(q), (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool),                        \
-                     block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu.data_ptr<int>(),                 \
-                     start.data_ptr<int>(), slp, gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr,      \
-                     gstride, H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap,     \
-                     sink ? 1 : 0)
+    const size_t msmem = (size_t)2 * MFMA_TILES_PER_STEP * (32 * (ds * 16 + 8) + vt * 32 * 40) * sizeof(bf16s);
+#define MFMA_CASE(DS_, VT_)                                                                                        \
+  do {                                                                                                             \
+    auto kfn = paged_attention_mfma_kernel<DS_, VT_>;                                                              \
+    if (msmem > 65536) /* more dynamic LDS than a kernel gets without asking */                                    \
+      (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)msmem);         \
+    hipLaunchKernelGGL(kfn, grid, dim3(64 * nw), msmem, stream(), ptr<bf16s>(out), ptr<bf16s>(q),                  \
+                       (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool), block_tables.data_ptr<int>(),      \
+                       (int)block_tables.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slp,                \
+                       gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr, gstride, H, G, D, Dv,         \
+                       page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap, sink ? 1 : 0);      \
+  } while (0)
 #define MFMA_ROW(DS_)                     \
   do {                                    \
     if (vt == 1) MFMA_CASE(DS_, 1);       \

@@ -52,7 +52,7 @@ def moe_config(s: dict, experts: int = 32, top: int = 6) -> MubutarConfig:
     inter = _inter(W)
     ff = W // 2
     shared = (3 * inter // 2 - top * ff + 127) // 128 * 128
-    att = dict(dim=D, heads=H, kv_heads=G, vdim=D, scale=D ** -0.5, softcap=50.0)
+    att = dict(dim=D, heads=H, kv_heads=G, vdim=D, scale=D ** -0.5, softcap=30.0)
     layers = []
     for i in range(s["layers"]):
         if i % 2 == 0:

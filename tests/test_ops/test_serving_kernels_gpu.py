@@ -218,7 +218,7 @@ def test_paged_attention_heads_per_block(counts):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("page", [16, 64])
-@pytest.mark.parametrize("H,G,D,Dv,cap", [(6, 2, 48, 96, 8.0), (4, 2, 40, 80, 0.0), (2, 1, 96, 72, 3.0), (8, 2, 64, 64, 50.0),
+@pytest.mark.parametrize("H,G,D,Dv,cap", [(6, 2, 48, 96, 8.0), (4, 2, 40, 80, 0.0), (2, 1, 96, 72, 3.0), (8, 2, 64, 64, 40.0),
                                           (3, 3, 24, 44, 5.0), (4, 4, 128, 128, 30.0), (4, 2, 16, 8, 1.0),
                                           (2, 2, 104, 120, 12.0)])
 def test_paged_attention_softcap_and_sink(dtype, H, G, D, Dv, cap, page):
