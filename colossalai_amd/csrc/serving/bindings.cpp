@@ -29,6 +29,9 @@ std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, at::Tensor correct
 at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at::Tensor ids, at::Tensor weights,
                            c10::optional<at::Tensor> base);
 at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base);
+std::vector<at::Tensor> expert_sort(at::Tensor ids, int64_t num_experts);
+at::Tensor expert_grouped_gemm(at::Tensor a, c10::optional<at::Tensor> a_rows, at::Tensor w, at::Tensor offsets,
+                               int64_t rows, bool relu_squared);
 
 }  // namespace serving
 }  // namespace cai
@@ -47,5 +50,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("add_rms_norm", &s::add_rms_norm, "residual += a (+ b) in place, then the RMS norm of the sum");
   m.def("grouped_topk_route", &s::grouped_topk_route, "sigmoid router: correction, group-limited top-k, renormalised");
   m.def("expert_ffn_gemv", &s::expert_ffn_gemv, "chosen experts' feed-forward of a small step, matrix-vector kernels");
+  m.def("expert_sort", &s::expert_sort, "stable sort of (token, expert) pairs by expert: offsets, source tokens, inverse");
+  m.def("expert_grouped_gemm", &s::expert_grouped_gemm,
+        "rows sorted by expert times their expert's matrix (bfloat16, MFMA), optional row gather and relu^2");
   m.def("expert_combine", &s::expert_combine, "base + weighted sum of each token's expert outputs, float32");
 }

@@ -5,8 +5,10 @@
 //                        (up + squared ReLU per (token, expert) pair, then the weighted
 //                        down products of a token summed with its base row) — only the
 //                        chosen experts' weights are streamed, nothing goes to the host;
+//   expert_sort        : stable counting sort of a step's (token, expert) pairs by expert,
+//                        one block, for the grouped matrix-core product (expert_gemm.hip);
 //   expert_combine     : base + weighted sum of each token's rows of a sorted-by-expert
-//                        output (the large-step path, whose products are library GEMMs).
+//                        output.
 #include "serving_common.h"
 
 namespace cai {
@@ -331,6 +333,79 @@ at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10:
 #undef COMBINE_LAUNCH
   HIP_CHECK_LAST();
   return out;
+}
+
+// ------------------------------------------------------------------- sort
+// Stable counting sort of the (token, expert) pairs of a step by expert, one block, the ids held in LDS:
+//   offsets[e] .. offsets[e + 1] = sorted rows of expert e; src[r] = token of sorted row r; inv[p] = sorted row of
+//   pair p. Each wave takes every nw-th expert and walks the pairs 64 at a time (ballot + prefix count), so rows of
+//   one expert keep the order of their pairs and the result does not depend on timing.
+constexpr int SORT_MAX_PAIRS = 8192;
+
+__global__ __launch_bounds__(1024) void expert_sort_kernel(
+    int* __restrict__ offsets, int* __restrict__ src, int* __restrict__ inv, const int* __restrict__ ids, int P, int E,
+    int top) {
+  extern __shared__ int sort_lds[];
+  int* held = sort_lds;          // [P]
+  int* count = sort_lds + P;     // [E + 1]
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  for (int p = threadIdx.x; p < P; p += blockDim.x) held[p] = ids[p];
+  __syncthreads();
+  for (int e = wid; e < E; e += nw) {
+    int n = 0;
+    for (int p0 = 0; p0 < P; p0 += 64) {
+      const bool hit = p0 + lane < P && held[p0 + lane] == e;
+      n += __popcll(__ballot(hit));
+    }
+    if (lane == 0) count[e] = n;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int n = count[e];
+      count[e] = run;
+      offsets[e] = run;
+      run += n;
+    }
+    count[E] = run;
+    offsets[E] = run;
+  }
+  __syncthreads();
+  for (int e = wid; e < E; e += nw) {
+    int at = count[e];
+    for (int p0 = 0; p0 < P; p0 += 64) {
+      const int p = p0 + lane;
+      const bool hit = p < P && held[p] == e;
+      const unsigned long long mask = __ballot(hit);
+      if (hit) {
+        const int r = at + __popcll(mask & ((1ull << lane) - 1ull));
+        src[r] = p / top;
+        inv[p] = r;
+      }
+      at += __popcll(mask);
+    }
+  }
+}
+
+std::vector<at::Tensor> expert_sort(at::Tensor ids, int64_t num_experts) {
+  check_i32(ids, "ids");
+  TORCH_CHECK(ids.dim() == 2, "ids must be [N, top]");
+  const int P = (int)ids.numel(), top = (int)ids.size(1), E = (int)num_experts;
+  TORCH_CHECK(P <= SORT_MAX_PAIRS, "too many pairs for the one-block sort");
+  TORCH_CHECK(E >= 1 && (size_t)(P + E + 1) * sizeof(int) <= 64 * 1024);
+  at::Tensor offsets = at::empty({E + 1}, ids.options());
+  at::Tensor src = at::empty({P}, ids.options());
+  at::Tensor inv = at::empty({ids.size(0), ids.size(1)}, ids.options());
+  if (P == 0) {
+    offsets.zero_();
+    return {offsets, src, inv};
+  }
+  // an id outside [0, E) would leave rows of src / inv unwritten: the router never produces one
+  hipLaunchKernelGGL(expert_sort_kernel, dim3(1), dim3(1024), (size_t)(P + E + 1) * sizeof(int), stream(),
+                     offsets.data_ptr<int>(), src.data_ptr<int>(), inv.data_ptr<int>(), ids.data_ptr<int>(), P, E, top);
+  HIP_CHECK_LAST();
+  return {offsets, src, inv};
 }
 
 }  // namespace serving

@@ -14,10 +14,14 @@ weights:
   index) and their plain scores are divided by their sum plus ``renorm_eps``.
 
 ``routed_expert_ffn`` runs ``down_e(act(up_e(h)))`` for each token's chosen
-experts and forms ``base + sum_j weight_j * y_j`` in float32. On the GPU a small
-step (decode tokens) streams just the chosen experts' weights through a
-matrix-vector kernel without touching the host; a large step (prompt portions)
-sorts the (token, expert) pairs by expert and runs one matrix product per expert.
+experts and forms ``base + sum_j weight_j * y_j`` in float32. On the GPU nothing
+of a bfloat16 step goes to the host: a small step (decode tokens) streams just
+the chosen experts' weights through matrix-vector kernels; a larger one sorts
+the (token, expert) pairs by expert on the device and runs each of the two
+products for all experts in one grouped matrix-core launch that reads the
+experts' row ranges from a device-side offsets vector. Float32 serving and
+sizes the grouped kernel does not tile take one library product per expert
+after a host-side count.
 """
 
 from typing import Optional
@@ -30,8 +34,13 @@ from .activation import relu_squared
 
 __all__ = ["grouped_topk_route", "grouped_topk_route_ref", "routed_expert_ffn", "routed_expert_ffn_ref"]
 
-# (token, expert) pairs up to which the matrix-vector kernels beat sorting + per-expert GEMMs
-GEMV_MAX_PAIRS = 256
+# (token, expert) pairs up to which the matrix-vector kernels are used (measured crossover, 32 experts of 1024 x
+# 2048: 66 against 84 us at 48 pairs, 95 against 88 us at 72): they re-read an expert's matrices (from cache) once
+# per pair and take two launches, the grouped product reads them once per 128 rows and takes four
+GEMV_MAX_PAIRS = 64
+# ... and where the grouped product does not apply (float32 serving, sizes it does not tile): up to here the
+# matrix-vector kernels beat the per-expert library products, whose launches and host round trip cost about 1.5 ms
+GEMV_FALLBACK_PAIRS = 2048
 
 
 def grouped_topk_route_ref(logits, correction, top: int, group_count: int = 1, group_keep: int = 1,
@@ -82,31 +91,61 @@ def routed_expert_ffn_ref(h, w_up, w_down, ids, weights, base=None, activation: 
     return out
 
 
-def _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation):
-    """Pairs sorted by expert, one up and one down product per expert that got
-    rows, then every token gathers its ``top`` results in slot order."""
-    N, top = ids.shape
-    E = w_up.shape[0]
+def _sort_pairs(ids, E: int):
+    """(order, inverse, offsets) of the (token, expert) pairs sorted by expert, all on the device: ``order[r]`` is
+    the pair at sorted row ``r`` (stable: ascending pair index inside an expert), ``offsets[e] .. offsets[e + 1]``
+    the rows of expert ``e``."""
     flat = ids.reshape(-1).long()
     order = torch.argsort(flat, stable=True)
-    counts = torch.bincount(flat, minlength=E).tolist()  # host: the products below are launched per expert
-    x = h.index_select(0, order // top)
-    hidden = torch.empty(x.shape[0], w_up.shape[1], dtype=h.dtype, device=h.device)
-    at = 0
-    for e, n in enumerate(counts):
-        if n:
-            torch.mm(x[at : at + n], w_up[e].t(), out=hidden[at : at + n])
-            at += n
-    hidden = _act(hidden, activation)
-    y = torch.empty(x.shape[0], w_down.shape[1], dtype=h.dtype, device=h.device)
-    at = 0
-    for e, n in enumerate(counts):
-        if n:
-            torch.mm(hidden[at : at + n], w_down[e].t(), out=y[at : at + n])
-            at += n
+    offsets = torch.zeros(E + 1, dtype=torch.int32, device=ids.device)
+    offsets[1:] = torch.cumsum(torch.bincount(flat, minlength=E), 0)
     inv = torch.empty_like(order)
     inv[order] = torch.arange(order.numel(), device=order.device)
+    return order, inv, offsets
+
+
+SORT_KERNEL_MAX_PAIRS = 8192  # the one-block sort kernel holds a step's ids in LDS
+
+
+def _grouped_expert_ffn(h, w_up, w_down, ids, weights, base):
+    """One grouped matrix-core launch per product; the up product gathers the tokens' rows itself and squares the
+    rectified accumulator. Steps of up to 8192 pairs are sorted by one kernel, larger ones by library sorts."""
+    N, top = ids.shape
+    K = serving_kernels()
+    if ids.numel() <= SORT_KERNEL_MAX_PAIRS:
+        offsets, src, inv = K.expert_sort(ids.contiguous(), w_up.shape[0])
+    else:
+        order, inv, offsets = _sort_pairs(ids, w_up.shape[0])
+        src, inv = (order // top).int(), inv.int().view(N, top)
+    hidden = K.expert_grouped_gemm(h, src, w_up, offsets, ids.numel(), True)
+    y = K.expert_grouped_gemm(hidden, None, w_down, offsets, ids.numel(), False)
+    return K.expert_combine(y, inv, weights, base)
+
+
+def _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation):
+    """Pairs sorted by expert, one up and one down library product per expert that got rows (their row counts come
+    to the host), then every token gathers its ``top`` results in slot order."""
+    N, top = ids.shape
+    order, inv, offsets = _sort_pairs(ids, w_up.shape[0])
+    bounds = offsets.tolist()
+    x = h.index_select(0, order // top)
+    hidden = torch.empty(x.shape[0], w_up.shape[1], dtype=h.dtype, device=h.device)
+    for e in range(w_up.shape[0]):
+        lo, hi = bounds[e], bounds[e + 1]
+        if hi > lo:
+            torch.mm(x[lo:hi], w_up[e].t(), out=hidden[lo:hi])
+    hidden = _act(hidden, activation)
+    y = torch.empty(x.shape[0], w_down.shape[1], dtype=h.dtype, device=h.device)
+    for e in range(w_up.shape[0]):
+        lo, hi = bounds[e], bounds[e + 1]
+        if hi > lo:
+            torch.mm(hidden[lo:hi], w_down[e].t(), out=y[lo:hi])
     return serving_kernels().expert_combine(y, inv.int().view(N, top), weights, base)
+
+
+def _grouped_fits(h, w_up, w_down) -> bool:
+    return (h.dtype == torch.bfloat16 and w_up.shape[2] % 32 == 0 and w_up.shape[1] % 32 == 0
+            and w_up.is_contiguous() and w_down.is_contiguous())
 
 
 def routed_expert_ffn(h, w_up, w_down, ids, weights, base: Optional[torch.Tensor] = None,
@@ -118,6 +157,11 @@ def routed_expert_ffn(h, w_up, w_down, ids, weights, base: Optional[torch.Tensor
         return routed_expert_ffn_ref(h, w_up, w_down, ids, weights, base, activation)
     if activation != "relu_squared":
         raise ValueError(f"unknown expert activation {activation!r}")
+    h = h.contiguous()
     if ids.numel() <= GEMV_MAX_PAIRS:
-        return serving_kernels().expert_ffn_gemv(h.contiguous(), w_up, w_down, ids, weights, base)
+        return serving_kernels().expert_ffn_gemv(h, w_up, w_down, ids, weights, base)
+    if _grouped_fits(h, w_up, w_down):
+        return _grouped_expert_ffn(h, w_up, w_down, ids, weights, base)
+    if ids.numel() <= GEMV_FALLBACK_PAIRS:
+        return serving_kernels().expert_ffn_gemv(h, w_up, w_down, ids, weights, base)
     return _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation)

@@ -151,14 +151,47 @@ def test_long_decode_over_many_pages(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_large_step_and_small_step_agree(device):
+def test_large_step_and_small_step_agree(device, monkeypatch):
     """A prompt long enough for the sorted per-expert products next to the
     same prompt decoded in small steps (matrix-vector experts on the GPU)."""
+    from colossalai_amd.ops import routed_experts
+
+    monkeypatch.setattr(routed_experts, "GEMV_MAX_PAIRS", 64)
+    monkeypatch.setattr(routed_experts, "GEMV_FALLBACK_PAIRS", 64)
     toks = prompt(120, 8)
     big = run_cut(engine(device), "a", toks, [120])
     small = run_cut(engine(device), "a", toks, [100] + [4] * 5)
     close(big, oracle(toks), 5e-4)
     close(small, oracle(toks), 5e-4)
+
+
+@pytest.mark.gpu
+def test_bfloat16_paths_agree_with_each_other_and_the_oracle():
+    """bfloat16 serving with sizes the matrix-core kernels tile: a whole prompt (grouped expert product, MFMA
+    attention) against the same prompt in small steps (matrix-vector experts, split-key attention)."""
+    att = dict(dim=32, heads=4, kv_heads=2, vdim=40, scale=0.18, softcap=6.0)
+    cfg = dict(architecture="Mubutar", vocab=64, width=64, embedding=dict(scale=2.0), logit_scale=1.0, norm=dict(eps=1e-5),
+               layers=[dict(type="attention", mixer=att,
+                            mlp=dict(kind="moe", expert=dict(ff=32), shared=dict(ff=32),
+                                     router=dict(experts=6, top=2, groups=dict(count=3, keep=2)))),
+                       dict(type="attention", mixer=dict(att, kv_from=0), mlp=dict(kind="dense", ff=96))])
+    W = {k: v.to(torch.bfloat16).float() for k, v in O.random_weights(cfg, seed=4).items()}
+    toks = torch.randint(0, 64, (70,), generator=torch.Generator().manual_seed(9)).tolist()
+    want = O.forward(cfg, W, toks).float()
+
+    def run(cuts):
+        model = MubutarForCausalLM.from_checkpoint(cfg, W, dtype=torch.bfloat16, device="cuda")
+        eng = ContinuousBatchEngine(model, InferenceConfig(max_batch_size=2, dtype=torch.bfloat16), num_blocks=16,
+                                    block_size=16)
+        return run_cut(eng, "a", toks, cuts).float().cpu()
+
+    whole, stepped = run([70]), run([40] + [3] * 10)
+    scale = want.pow(2).mean().sqrt()
+    for got in (whole, stepped):
+        err = (got - want).pow(2).mean(-1).sqrt() / scale
+        assert err.median().item() < 0.03 and (err < 0.1).float().mean().item() > 0.8
+    both = (whole - stepped).pow(2).mean(-1).sqrt() / scale
+    assert both.median().item() < 0.03
 
 
 @pytest.mark.parametrize("device", DEVICES)

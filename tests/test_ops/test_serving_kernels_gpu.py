@@ -302,9 +302,13 @@ def test_grouped_topk_route(E, top, groups, keep):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("N,W,Fe,E,top,shared", [(7, 256, 96, 8, 2, True), (3, 100, 36, 5, 3, False), (1, 512, 200, 4, 4, True),
-                                               (300, 256, 128, 6, 2, True), (200, 96, 40, 16, 1, False)])
+                                               (300, 256, 128, 6, 2, True), (200, 96, 40, 16, 1, False),
+                                               (700, 64, 32, 6, 2, True), (1100, 40, 24, 3, 1, False),
+                                               (2200, 40, 24, 3, 1, False), (900, 160, 96, 40, 4, True)])
 def test_routed_expert_ffn(dtype, N, W, Fe, E, top, shared):
-    """Few pairs: matrix-vector kernels; many: sorted per-expert products and the combine kernel."""
+    """Few pairs: matrix-vector kernels. Many: in bfloat16 with sizes that are multiples of 32 the grouped
+    matrix-core product (device-side sort, no host round trip), else matrix-vector kernels again and, past their
+    limit, sorted per-expert library products."""
     torch.manual_seed(13)
     h = torch.randn(N, W).to(dtype)
     w_up = (torch.randn(E, Fe, W) / W ** 0.5).to(dtype)
@@ -319,3 +323,44 @@ def test_routed_expert_ffn(dtype, N, W, Fe, E, top, shared):
     assert out.dtype == torch.float32
     torch.testing.assert_close(out.cpu(), ref, **(dict(rtol=3e-2, atol=3e-2) if dtype == torch.bfloat16
                                                   else dict(rtol=1e-4, atol=1e-4)))
+
+
+@pytest.mark.parametrize("M,K", [(128, 64), (96, 32), (200, 160), (384, 1024)])
+def test_expert_grouped_gemm(M, K):
+    """Row ranges of very different sizes, experts without rows at both ends and in the middle, output widths that
+    are no multiple of the tile, with and without the row gather and the squared-ReLU epilogue."""
+    from colossalai_amd.ops._kernels import serving_kernels
+
+    torch.manual_seed(14)
+    counts = [0, 5, 0, 300, 1, 129, 0, 128, 64, 0]
+    E, P = len(counts), sum(counts)
+    offsets = torch.tensor([0] + torch.tensor(counts).cumsum(0).tolist(), dtype=torch.int32)
+    w = (torch.randn(E, M, K) / K ** 0.5).bfloat16()
+    src_rows = torch.randint(0, 50, (P,), dtype=torch.int32)
+    a_small, a_full = torch.randn(50, K).bfloat16(), torch.randn(P, K).bfloat16()
+    for a, rows, act in ((a_small, src_rows, True), (a_full, None, False)):
+        out = serving_kernels().expert_grouped_gemm(a.cuda(), None if rows is None else rows.cuda(), w.cuda(),
+                                                    offsets.cuda(), P, act)
+        x = a.float() if rows is None else a.float()[rows.long()]
+        ref = torch.empty(P, M)
+        for e in range(E):
+            lo, hi = int(offsets[e]), int(offsets[e + 1])
+            ref[lo:hi] = x[lo:hi] @ w[e].float().t()
+        if act:
+            ref = torch.relu(ref).square()
+        torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("N,top,E", [(1, 1, 1), (40, 3, 7), (1000, 6, 32), (2048, 4, 200), (77, 1, 3)])
+def test_expert_sort(N, top, E):
+    from colossalai_amd.ops._kernels import serving_kernels
+
+    torch.manual_seed(15)
+    ids = torch.randint(0, E, (N, top), dtype=torch.int32)
+    if E > 2:
+        ids[ids == 1] = 2  # an expert without rows
+    offsets, src, inv = (t.cpu() for t in serving_kernels().expert_sort(ids.cuda(), E))
+    order, inv_ref, offsets_ref = routed_experts._sort_pairs(ids, E)
+    assert offsets.tolist() == offsets_ref.tolist()
+    assert src.tolist() == (order // top).tolist()
+    assert inv.reshape(-1).tolist() == inv_ref.tolist()
