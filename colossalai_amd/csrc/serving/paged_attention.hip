@@ -363,7 +363,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
   };
 
-  float m = -INFINITY, l = 0.0f;  // m in the base-2 domain
+  // With a sink and a soft cap the scores live in [-cap2, cap2] (a distance penalty only lowers them) and the
+  // denominator holds the sink's exp2(0) = 1: the weights can be taken against the fixed reference 0 instead of a
+  // running maximum. exp2(cap2) cannot overflow for cap2 <= 96, and a weight that underflows is nothing beside the
+  // sink's 1. No maximum to track, no accumulator to rescale.
+  const bool fixed_ref = sink != 0 && softcap > 0.0f && softcap * 1.4426950408889634f <= 96.0f;
+  float m = fixed_ref ? 0.0f : -INFINITY, l = 0.0f;  // m in the base-2 domain
   f32x16 oacc[VT];
 #pragma unroll
   for (int t = 0; t < VT; ++t)
@@ -415,7 +420,6 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       }
       // scores in the base-2 domain: s2 = (q.k) scale log2e - slope log2e (pos - j), one add and one fma each
       float sv[16];
-      float tmax = -INFINITY;
       const float tile_bias = -sl2 * (float)(pos - kbase);
       // interior tile: every key is visible to every token of the tile, no masks to evaluate
       const bool interior = !sink && t_off + 31 < cnt && kbase + 31 <= p0 && (window == 0 || p1 - kbase < window);
@@ -423,7 +427,6 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           sv[i] = base2(sacc[i]) + (tile_bias + row_bias[i]);
-          tmax = fmaxf(tmax, sv[i]);
         }
       } else {
 #pragma unroll
@@ -431,13 +434,19 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
           const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
           const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
           sv[i] = seen ? base2(sacc[i]) + (tile_bias + row_bias[i]) : -INFINITY;
-          tmax = fmaxf(tmax, sv[i]);
         }
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-      const float m_new = fmaxf(m, tmax);
-      const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: every weight is exp2(-inf) = 0
-      const float corr = (m == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - m_new);  // nothing accumulated: nothing to rescale
+      float m_ref = 0.0f, corr = 1.0f;
+      if (!fixed_ref) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, sv[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float m_new = fmaxf(m, tmax);
+        m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // nothing visible yet: every weight is exp2(-inf) = 0
+        corr = (m == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - m_new);  // nothing accumulated: nothing to rescale
+        m = m_new;
+      }
       float psum = 0.0f;
       bf16x8_v phi[2], plo[2];
 #pragma unroll
@@ -449,8 +458,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         plo[i >> 3][i & 7] = (__bf16)(p - (float)hi);
       }
       l = l * corr + psum;
-      m = m_new;
-      if (!__all(corr == 1.0f)) {  // the running maxima of all 32 tokens stood still: no rescaling
+      if (!fixed_ref && !__all(corr == 1.0f)) {  // the running maxima of all 32 tokens stood still: no rescaling
 #pragma unroll
         for (int t = 0; t < VT; ++t)
 #pragma unroll

@@ -249,6 +249,27 @@ def test_paged_attention_softcap_and_sink(dtype, H, G, D, Dv, cap, page):
                                **loose)
 
 
+@pytest.mark.parametrize("cap", [2.0, 60.0, 66.0, 70.0])
+def test_saturated_softcap_with_sink(cap):
+    """Scores pushed against both ends of the cap. With a sink and a cap the matrix-core kernel takes its
+    weights against the fixed reference 0 as long as exp2 of the cap cannot overflow (cap <= 66.5) and against
+    a running maximum beyond; either way keys at -cap vanish beside keys at +cap and beside the sink."""
+    torch.manual_seed(16)
+    H, G, D, Dv, page = 4, 2, 64, 64, 16
+    gb, cb, pages = make_batch("cuda", page)
+    N = gb.num_tokens
+    kpool, vpool = torch.randn(pages, page, G, D).bfloat16(), torch.randn(pages, page, G, Dv).bfloat16()
+    kg, vg = kpool.cuda(), vpool.cuda()
+    q, k, v = (torch.randn(N, H, D) * 40).bfloat16(), torch.randn(N, G, D).bfloat16(), torch.randn(N, G, Dv).bfloat16()
+    q[::3] = -q[::3].abs() * k[::3].repeat_interleave(H // G, 1).sign()   # these tokens score themselves near -cap
+    paged_attention.paged_kv_write(k.cuda(), v.cuda(), kg, vg, gb)
+    paged_attention.paged_kv_write(k, v, kpool, vpool, cb)
+    out = paged_attention.paged_attention(q.cuda(), kg, vg, gb, 1.0, softcap=cap, sink=True)
+    ref = paged_attention.paged_attention_ref(q, kpool, vpool, cb, 1.0, softcap=cap, sink=True)
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=3e-2, atol=3e-2)
+
+
 def test_sink_with_tiny_scores_halves_nothing_by_accident():
     """Scores of exactly 0 for t visible keys: every weight is 1 / (t + 1)."""
     page, T, D, Dv = 16, 40, 32, 32
