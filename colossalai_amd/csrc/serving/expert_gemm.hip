@@ -20,6 +20,7 @@ namespace cai {
 namespace serving {
 
 constexpr int GG_TM = 128, GG_TN = 128, GG_TK = 32, GG_PITCH = GG_TK + 8;
+constexpr int GG_MAX_EXPERTS = 1024;
 
 template <bool RELU_SQ>
 __global__ __launch_bounds__(256) void expert_grouped_gemm_kernel(
@@ -28,11 +29,15 @@ __global__ __launch_bounds__(256) void expert_grouped_gemm_kernel(
   __shared__ __align__(16) bf16s As[2][GG_TM * GG_PITCH];
   __shared__ __align__(16) bf16s Bs[2][GG_TN * GG_PITCH];
   const int tid = threadIdx.x, wid = tid >> 6, lane = tid & 63;
-  // which expert and which of its row tiles
+  // which expert and which of its row tiles: the offsets come into LDS with one load per thread, every thread then
+  // walks them there
+  __shared__ int offs[GG_MAX_EXPERTS + 1];
+  for (int i = tid; i <= E; i += 256) offs[i] = offsets[i];
+  __syncthreads();
   int t = blockIdx.x, e = 0, row0 = 0, row_end = 0;
   bool found = false;
   for (; e < E; ++e) {
-    const int lo = offsets[e], hi = offsets[e + 1];
+    const int lo = offs[e], hi = offs[e + 1];
     const int nt = (hi - lo + GG_TM - 1) / GG_TM;
     if (t < nt) {
       row0 = lo + t * GG_TM;
@@ -138,6 +143,7 @@ at::Tensor expert_grouped_gemm(at::Tensor a, c10::optional<at::Tensor> a_rows, a
   const int E = (int)w.size(0), M = (int)w.size(1), K = (int)w.size(2);
   TORCH_CHECK(a.size(1) == K && offsets.numel() == E + 1, "shapes of a / w / offsets do not fit");
   TORCH_CHECK(K % GG_TK == 0, "the contraction size must be a multiple of 32");
+  TORCH_CHECK(E <= GG_MAX_EXPERTS, "more experts than the grouped product's offsets buffer holds");
   TORCH_CHECK(reinterpret_cast<uintptr_t>(a.data_ptr()) % 16 == 0 && reinterpret_cast<uintptr_t>(w.data_ptr()) % 16 == 0);
   const int* rows_ptr = nullptr;
   if (a_rows.has_value()) {

@@ -145,7 +145,7 @@ def _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation):
 
 def _grouped_fits(h, w_up, w_down) -> bool:
     return (h.dtype == torch.bfloat16 and w_up.shape[2] % 32 == 0 and w_up.shape[1] % 32 == 0
-            and w_up.is_contiguous() and w_down.is_contiguous())
+            and w_up.shape[0] <= 1024 and w_up.is_contiguous() and w_down.is_contiguous())
 
 
 def routed_expert_ffn(h, w_up, w_down, ids, weights, base: Optional[torch.Tensor] = None,
