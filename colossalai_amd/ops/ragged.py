@@ -72,15 +72,23 @@ class RaggedBatch:
                 t = tables[i]
                 assert len(t) * page_size >= starts[i] + n, "block table does not cover the new tokens"
                 rows += [t[p // page_size] * page_size + p % page_size for p in range(starts[i], starts[i] + n)]
-        i32 = dict(dtype=torch.int32, device=device)
-        bt = None
+        # one host-to-device copy for all index vectors of the step; the fields are views into it
+        B = len(new_counts)
+        parts = [cu, list(starts), list(slots), tok_seq, pos]
+        width = 0
         if tables is not None:
             width = max(len(t) for t in tables)
-            bt = torch.tensor([list(t) + [0] * (width - len(t)) for t in tables], **i32)
+            parts += [[p for t in tables for p in list(t) + [0] * (width - len(t))], rows]
+        flat = [v for part in parts for v in part]
+        buf = torch.tensor(flat, dtype=torch.int32).to(device)
+        sizes = [len(part) for part in parts]
+        views, at = [], 0
+        for n in sizes:
+            views.append(buf[at : at + n])
+            at += n
         return cls(
-            cu=torch.tensor(cu, **i32), start=torch.tensor(list(starts), **i32),
-            slots=torch.tensor(list(slots), **i32), tok_seq=torch.tensor(tok_seq, **i32),
-            positions=torch.tensor(pos, **i32), block_tables=bt,
-            kv_rows=torch.tensor(rows, **i32) if tables is not None else None,
+            cu=views[0], start=views[1], slots=views[2], tok_seq=views[3], positions=views[4],
+            block_tables=views[5].view(B, width) if tables is not None else None,
+            kv_rows=views[6] if tables is not None else None,
             cu_host=cu, start_host=list(starts), slots_host=list(slots), page_size=page_size,
         )
