@@ -40,7 +40,11 @@ DEV_INLINE float reduce8(float v) { return dpp_add<0x141>(dpp_add<0x4E>(dpp_add<
 // Values: lane = a pair of value channels, the block's weights and pool rows come from LDS.
 // RC = query heads per block: 4 shares each key/value read between the most heads; 2 or 1 are
 // chosen when a decode step would otherwise leave most CUs without a block (the re-reads hit L2).
-template <typename T, int RC>
+// V8 (value head sizes 8, 16, ..., 256): a lane takes 8 consecutive value channels of a key with one 16/32-byte
+// load, Dv / 8 lanes cover a key's row and the 64 / (Dv / 8) lane groups take different keys of the block, so a
+// block of 64 keys is read by Dv / 8 load instructions instead of 64; the groups' sums meet in a butterfly of
+// shuffles after the last block.
+template <typename T, int RC, bool V8>
 __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_seq,
@@ -81,14 +85,19 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
   const int DS = (((D + 7) >> 3) + 7) & ~7;  // slice of the head size per lane, a multiple of 8
   const int d_lo = part8 * DS, d_hi = min(D, d_lo + DS);
 
-  float m[RC], l[RC], acc[RC][4];
+  constexpr int NA = V8 ? 8 : 4;  // value channels a lane accumulates
+  float m[RC], l[RC], acc[RC][NA];
 #pragma unroll
   for (int r = 0; r < RC; ++r) {
     m[r] = -INFINITY;
     l[r] = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
+    for (int i = 0; i < NA; ++i) acc[r][i] = 0.0f;
   }
+  const int vl = Dv >> 3;                     // V8: lanes per key row (a power of two) ...
+  const int vks = V8 ? 64 / vl : 1;           // ... keys per load instruction ...
+  const int vsub = V8 ? lane / vl : 0;        // ... this lane's key group ...
+  const int vch = V8 ? (lane % vl) * 8 : 0;   // ... and its first value channel
 
   for (int base = wid * 64; base < total; base += 64 * nw) {
     const int cnt = min(64, total - base);
@@ -155,7 +164,20 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
 #pragma unroll
     for (int r = 0; r < RC; ++r)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[r][i] *= corr[r];
+      for (int i = 0; i < NA; ++i) acc[r][i] *= corr[r];
+    if constexpr (V8) {
+#pragma unroll 4
+      for (int jj = vsub; jj < cnt; jj += vks) {
+        float v[8];
+        load8(vpool + ((long)prow[jj] * G + g) * Dv + vch, v);
+#pragma unroll
+        for (int r = 0; r < RC; ++r) {
+          const float w = pw[r * 64 + jj];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[r][e] += w * v[e];
+        }
+      }
+    } else {
     const int dva = 2 * lane, dvb = 128 + 2 * lane;
 #pragma unroll 8
     for (int jj = 0; jj < cnt; ++jj) {
@@ -176,6 +198,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
         acc[r][0] += w * v0; acc[r][1] += w * v1; acc[r][2] += w * v2; acc[r][3] += w * v3;
       }
     }
+    }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
   const int PS = 2 + Dv;
@@ -183,11 +206,20 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
 #pragma unroll
   for (int r = 0; r < RC; ++r) {
     if (lane == 0) { mine[r * PS] = m[r]; mine[r * PS + 1] = l[r]; }
-    const int dva = 2 * lane, dvb = 128 + 2 * lane;
-    if (dva < Dv) mine[r * PS + 2 + dva] = acc[r][0];
-    if (dva + 1 < Dv) mine[r * PS + 2 + dva + 1] = acc[r][1];
-    if (dvb < Dv) mine[r * PS + 2 + dvb] = acc[r][2];
-    if (dvb + 1 < Dv) mine[r * PS + 2 + dvb + 1] = acc[r][3];
+    if constexpr (V8) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = acc[r][e];
+        for (int off = vl; off < 64; off <<= 1) v += __shfl_xor(v, off);  // the key groups' sums of this channel
+        if (vsub == 0) mine[r * PS + 2 + vch + e] = v;
+      }
+    } else {
+      const int dva = 2 * lane, dvb = 128 + 2 * lane;
+      if (dva < Dv) mine[r * PS + 2 + dva] = acc[r][0];
+      if (dva + 1 < Dv) mine[r * PS + 2 + dva + 1] = acc[r][1];
+      if (dvb < Dv) mine[r * PS + 2 + dvb] = acc[r][2];
+      if (dvb + 1 < Dv) mine[r * PS + 2 + dvb + 1] = acc[r][3];
+    }
   }
   __syncthreads();
   for (int i = threadIdx.x; i < nh * Dv; i += blockDim.x) {
@@ -580,19 +612,25 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
   const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
   const int vvec = Dv % 2 == 0 ? 1 : 0;
+  // value rows of 8, 16, ..., 256 channels whose loads are aligned take the 8-channels-per-lane value phase
+  const bool v8 = Dv >= 8 && (Dv & (Dv - 1)) == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0;
 #define SCALAR_CASE(RC_)                                                                                            \
-  hipLaunchKernelGGL((paged_attention_kernel<T, RC_>), dim3((unsigned)(N * G * chunks)), dim3(64 * nwaves), smem,   \
+  if (v8) SCALAR_LAUNCH(RC_, true);                                                                                 \
+  else SCALAR_LAUNCH(RC_, false)
+#define SCALAR_LAUNCH(RC_, V8_)                                                                                     \
+  hipLaunchKernelGGL((paged_attention_kernel<T, RC_, V8_>), dim3((unsigned)(N * G * chunks)), dim3(64 * nwaves), smem,   \
                      stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),             \
                      block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),            \
                      positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride, \
                      H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec,                \
                      (float)softcap, sink ? 1 : 0)
   SERVING_DISPATCH_ACT(q, T, {
-    if (rc == 4) SCALAR_CASE(4);
-    else if (rc == 2) SCALAR_CASE(2);
-    else SCALAR_CASE(1);
+    if (rc == 4) { SCALAR_CASE(4); }
+    else if (rc == 2) { SCALAR_CASE(2); }
+    else { SCALAR_CASE(1); }
   });
 #undef SCALAR_CASE
+#undef SCALAR_LAUNCH
   HIP_CHECK_LAST();
   return out;
 }
